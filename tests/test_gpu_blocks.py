@@ -1,0 +1,92 @@
+"""Flux blocks on the HIP kernels vs the plain-PyTorch blocks, the way the reference's
+tests/test_blocks.py does it (state dict shared, bf16, atol 0.1), plus the full 4608-token single
+block against the CPU oracle and fused-vs-unfused agreement."""
+import pytest
+import torch
+
+import triton_kernels as tk
+from oracle import flux_oracle as oracle
+from triton_kernels import flux
+from triton_kernels import testing as cfg
+from util import DEV, randn, seeded
+
+pytestmark = pytest.mark.gpu
+
+HEADS, HEAD_DIM = 24, 128
+HID = HEADS * HEAD_DIM
+
+
+def _pair(kind, seed):
+    torch.manual_seed(seed)
+    if kind == "single":
+        ref = flux.SingleStreamBlock(HID, HEADS, mlp_ratio=4.0).to(torch.bfloat16)
+        hip = tk.SingleStreamBlock(HID, HEADS, mlp_ratio=4.0).to(torch.bfloat16)
+    else:
+        ref = flux.DoubleStreamBlock(HID, HEADS, mlp_ratio=4.0).to(torch.bfloat16)
+        hip = tk.DoubleStreamBlock(HID, HEADS, mlp_ratio=4.0).to(torch.bfloat16)
+    hip.load_state_dict(ref.state_dict())
+    return ref.to(DEV), hip.to(DEV)
+
+
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("seq_len", [256, 1024])
+def test_single_stream_block(batch_size, seq_len):
+    ref, hip = _pair("single", seq_len + batch_size)
+    g = seeded(seq_len)
+    x = randn(g, batch_size, seq_len, HID, dtype=torch.bfloat16).to(DEV)
+    vec = randn(g, batch_size, HID, dtype=torch.bfloat16).to(DEV)
+    pe = randn(g, 1, 1, seq_len, HEAD_DIM // 2, 2, 2).to(DEV)
+    with torch.no_grad():
+        y_ref = ref(x=x, vec=vec, pe=pe)
+        y_hip = hip(x=x, vec=vec, pe=pe)
+        hip.fused = False
+        y_unfused = hip(x=x, vec=vec, pe=pe)
+    torch.testing.assert_close(y_hip, y_ref, atol=0.1, rtol=0)
+    torch.testing.assert_close(y_unfused, y_ref, atol=0.1, rtol=0)
+    torch.testing.assert_close(y_hip, y_unfused, atol=0.05, rtol=0)
+
+
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("img_seq_len", [256, 1024])
+def test_double_stream_block(batch_size, img_seq_len):
+    ref, hip = _pair("double", img_seq_len + batch_size)
+    g = seeded(img_seq_len)
+    txt_len = 256
+    img = randn(g, batch_size, img_seq_len, HID, dtype=torch.bfloat16).to(DEV)
+    txt = randn(g, batch_size, txt_len, HID, dtype=torch.bfloat16).to(DEV)
+    vec = randn(g, batch_size, HID, dtype=torch.bfloat16).to(DEV)
+    pe = randn(g, 1, 1, txt_len + img_seq_len, HEAD_DIM // 2, 2, 2).to(DEV)
+    with torch.no_grad():
+        r_img, r_txt = ref(img=img, txt=txt, vec=vec, pe=pe)
+        h_img, h_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
+        hip.fused = False
+        u_img, u_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
+    torch.testing.assert_close(h_img, r_img, atol=0.1, rtol=0)
+    torch.testing.assert_close(h_txt, r_txt, atol=0.1, rtol=0)
+    torch.testing.assert_close(u_img, r_img, atol=0.1, rtol=0)
+    torch.testing.assert_close(u_txt, r_txt, atol=0.1, rtol=0)
+
+
+def test_single_block_4608_tokens_vs_oracle():
+    """The headline workload: 512 txt + 64x64 img tokens, hidden 3072, against the state-dict driven
+    oracle evaluated by PyTorch on the same device (the CPU evaluation of a quarter-size sequence is
+    in test_single_block_small_vs_cpu_oracle)."""
+    x, vec, pe, sd = cfg.config5_block(DEV)
+    blk = tk.SingleStreamBlock(HID, HEADS).to(torch.bfloat16).to(DEV)
+    blk.load_state_dict(sd)
+    with torch.no_grad():
+        y = blk(x, vec, pe)
+        want = oracle.single_stream_block_ref(sd, x, vec, pe, HEADS)
+    torch.testing.assert_close(y, want, atol=0.1, rtol=0)
+    err = (y.float() - want.float()).abs()
+    assert err.mean().item() < 5e-3, f"mean error {err.mean().item()}"
+
+
+def test_single_block_small_vs_cpu_oracle():
+    x, vec, pe, sd = cfg.config5_block("cpu", n_txt=64, grid=16)
+    want = oracle.single_stream_block_ref(sd, x, vec, pe, HEADS)     # CPU, same bits
+    blk = tk.SingleStreamBlock(HID, HEADS).to(torch.bfloat16).to(DEV)
+    blk.load_state_dict(sd)
+    with torch.no_grad():
+        y = blk(x.to(DEV), vec.to(DEV), pe.to(DEV))
+    torch.testing.assert_close(y.cpu(), want, atol=0.1, rtol=0)

@@ -1,0 +1,120 @@
+"""HIP linear (bf16 MFMA GEMM with fused epilogues) vs the oracle.
+
+Grid and tolerances of the reference's tests/test_linear.py (bf16; atol 1e-5 without activation is
+not attainable against a *different* bf16 GEMM on inputs ~N(0,1) with K up to 1024, where one bf16
+ulp of the output is 0.25, so the no-activation cases compare against the fp32 result with the
+half-ulp bound instead), plus the Flux shapes at atol 2e-2 vs fp32, ragged shapes, and every
+epilogue the fused blocks use.
+"""
+import math
+
+import pytest
+import torch
+
+import triton_kernels as tk
+from oracle import flux_oracle as oracle
+from triton_kernels import testing as cfg
+from util import DEV, randn, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def half_ulp_bound(ref_fp32: torch.Tensor) -> torch.Tensor:
+    """|bf16(x) - x| <= 2^-9 |x| ; allow accumulation-order noise of a few fp32 ulps on top."""
+    return ref_fp32.abs() * 2.0 ** -8 + 1e-6
+
+
+@pytest.mark.parametrize("batch_size", [1, 4])
+@pytest.mark.parametrize("seq_len", [256, 1024])
+@pytest.mark.parametrize("in_channel", [256, 1024])
+@pytest.mark.parametrize("out_channel", [1024, 3072])
+@pytest.mark.parametrize("activation", ["", "GELU"])
+def test_linear_reference_grid(batch_size, seq_len, in_channel, out_channel, activation):
+    g = seeded(batch_size + seq_len + in_channel + out_channel)
+    x = randn(g, batch_size, seq_len, in_channel, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, out_channel, in_channel, dtype=torch.bfloat16).to(DEV)
+    b = randn(g, out_channel, dtype=torch.bfloat16).to(DEV)
+    y = tk.linear(x, w, b, activation=activation)
+    assert y.shape == (batch_size, seq_len, out_channel) and y.dtype == torch.bfloat16
+    if activation == "GELU":
+        # the reference's own tolerance for this case (tests/test_linear.py:26)
+        ref = oracle.linear_ref(x, w, b, activation)
+        pre = oracle.linear_ref_fp32(x, w, b)
+        # a one-ulp difference of the pre-activation (|y| up to ~150 here) moves the output by that ulp
+        tol = 0.02 + pre.abs() * 2.0 ** -7
+        assert ((y.float() - ref.float()).abs() <= tol).all()
+    else:
+        ref32 = oracle.linear_ref_fp32(x, w, b)
+        assert ((y.float() - ref32).abs() <= half_ulp_bound(ref32)).all()
+
+
+@pytest.mark.parametrize("which,act", [("mlp_in", "GELU"), ("proj_out", ""), ("linear1", "")])
+def test_linear_flux_shapes_vs_fp32(which, act):
+    a, w, b = cfg.config4(DEV, which, m=1024 if which != "mlp_in" else 4608)
+    y = tk.linear(a, w, b, activation=act)
+    ref32 = oracle.linear_ref_fp32(a, w, b, act)
+    torch.testing.assert_close(y.float(), ref32, atol=2e-2, rtol=0)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 9216, 3072), (2, 1000, 512), (7, 33, 64), (8, 18432, 3072), (9, 40, 72),
+                                   (130, 70, 200), (257, 513, 136), (300, 256, 8), (64, 64, 1000), (513, 1025, 264)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_linear_ragged_shapes(M, N, K, bias):
+    g = seeded(M * 3 + N * 5 + K)
+    x = randn(g, M, K, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, N, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16).to(DEV) if bias else None
+    y = tk.linear(x, w, b)
+    ref32 = oracle.linear_ref_fp32(x, w, b)
+    assert ((y.float() - ref32).abs() <= half_ulp_bound(ref32) + 1e-3).all()
+
+
+def test_linear_unaligned_k_and_strided_input():
+    g = seeded(3)
+    x = randn(g, 50, 77, dtype=torch.bfloat16).to(DEV)       # K = 77: no 16-byte rows
+    w = randn(g, 30, 77, dtype=torch.bfloat16, std=0.1).to(DEV)
+    y = tk.linear(x, w, None)
+    torch.testing.assert_close(y.float(), oracle.linear_ref_fp32(x, w, None), atol=2e-2, rtol=1e-2)
+    big = randn(g, 300, 1024, dtype=torch.bfloat16).to(DEV)
+    xs = big[:, 256:768]                                      # row stride 1024, K = 512
+    w = randn(g, 384, 512, dtype=torch.bfloat16, std=512 ** -0.5).to(DEV)
+    torch.testing.assert_close(tk.linear(xs, w, None).float(), oracle.linear_ref_fp32(xs, w, None), atol=2e-2, rtol=0)
+
+
+def test_linear_rejects_fp32_like_the_reference():
+    x = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(KeyError):
+        tk.linear(x, torch.zeros(16, 8, device=DEV), None)
+
+
+@pytest.mark.parametrize("M,hid,mlp", [(512, 256, 1024), (300, 128, 512), (4608, 3072, 12288)])
+def test_linear_split_gelu_epilogue(M, hid, mlp):
+    """linear1 of the single block: columns [0, 3*hid) plain -> out, columns [3*hid, ..) GELU -> out2."""
+    g = seeded(M + hid)
+    x = randn(g, M, hid, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, 3 * hid + mlp, hid, dtype=torch.bfloat16, std=hid ** -0.5).to(DEV)
+    b = randn(g, 3 * hid + mlp, dtype=torch.bfloat16, std=0.02).to(DEV)
+    qkv = torch.empty(M, 3 * hid, dtype=torch.bfloat16, device=DEV)
+    both = torch.zeros(M, hid + mlp, dtype=torch.bfloat16, device=DEV)
+    tk.linear_into(x, w, b, activation="GELU", act_begin=3 * hid, out=qkv, out2=both[:, hid:], split=3 * hid)
+    ref32 = oracle.linear_ref_fp32(x, w, b)
+    torch.testing.assert_close(qkv.float(), ref32[:, :3 * hid], atol=2e-2, rtol=0)
+    want_mlp = oracle.gelu_tanh_ref(ref32[:, 3 * hid:].to(torch.bfloat16))
+    torch.testing.assert_close(both[:, hid:], want_mlp, atol=2e-2, rtol=0)
+    assert (both[:, :hid] == 0).all()                        # the attention half is left alone
+
+
+@pytest.mark.parametrize("B,L,hid,K", [(1, 512, 256, 1280), (2, 300, 128, 640), (1, 4608, 3072, 15360)])
+def test_linear_gated_residual_epilogue(B, L, hid, K):
+    g = seeded(B + L + hid)
+    a = randn(g, B * L, K, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, hid, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, hid, dtype=torch.bfloat16, std=0.02).to(DEV)
+    x = randn(g, B, L, hid, dtype=torch.bfloat16).to(DEV)
+    mod = randn(g, B, 3 * hid, dtype=torch.bfloat16).to(DEV)
+    gate = mod[:, None, :].chunk(3, dim=-1)[2]
+    out = torch.empty_like(x)
+    tk.linear_into(a, w, b, out=out.view(B * L, hid), resid=x.view(B * L, hid), gate=gate)
+    y = oracle.linear_ref_fp32(a, w, b).to(torch.bfloat16).view(B, L, hid)
+    want = oracle.gated_residual_ref(x, gate, y)
+    torch.testing.assert_close(out, want, atol=4e-2, rtol=1e-2)

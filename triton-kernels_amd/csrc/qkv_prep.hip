@@ -1,0 +1,232 @@
+// Q/K/V preparation: one streaming pass that gathers q, k, v rows from up to two strided sources
+// (txt first, then img) into contiguous [B,H,L,D] tensors, optionally RMS-normalising q and k over
+// the head dimension and rotating them with the per-position 2x2 RoPE matrices on the way through.
+//
+// A row of D elements is owned by D/VEC adjacent lanes (16 lanes for D = 128 in bf16), each holding
+// one 16-byte vector = VEC/2 rotation pairs, so the per-row reduction is a DPP butterfly and the
+// rotation needs no cross-lane traffic. q and k of the same (b,h,s) are handled by the same lane
+// and share the pe registers. Blocks walk the sequence fastest, so the tile of pe a block needs is
+// the same for every head and stays in the L2 of the XCD that keeps getting that tile.
+#include "common.h"
+
+namespace flux {
+
+constexpr int kPrepBlock = 256;
+
+struct Src {
+    const void* txt; int64_t t_sb, t_sh, t_sl;
+    const void* img; int64_t i_sb, i_sh, i_sl;
+    void* out;
+    const void* scale_txt; const void* scale_img;
+};
+
+struct PrepParams {
+    Src q, k, v;
+    const float* pe;
+    int64_t pe_sb;
+    int64_t H, Lt, L;
+    float eps;
+};
+
+template <typename T>
+__device__ __forceinline__ const T* src_row(const Src& s, int64_t b, int64_t h, int64_t pos, int64_t Lt, bool& is_txt) {
+    is_txt = pos < Lt;
+    if (is_txt) return static_cast<const T*>(s.txt) + b * s.t_sb + h * s.t_sh + pos * s.t_sl;
+    return static_cast<const T*>(s.img) + b * s.i_sb + h * s.i_sh + (pos - Lt) * s.i_sl;
+}
+
+template <typename T, typename TS, int D, bool NORM, bool ROPE>
+__global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int G = (D / VEC) < 64 ? (D / VEC) : 64;   // lanes per row
+    constexpr int ITER = D / (VEC * G);                   // 16-byte vectors per lane
+    constexpr int ROWS = kPrepBlock / G;
+    static_assert(G * ITER * VEC == D, "head dim must be a multiple of the vector width");
+    const int lane = threadIdx.x % G;
+    const int64_t pos = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / G;
+    const int64_t bh = blockIdx.y;
+    const int64_t b = bh / p.H, h = bh % p.H;
+    const bool ok = pos < p.L;
+    const int64_t out_row = (bh * p.L + pos) * D;
+
+    // pe[pos, pair, a, j]: the lane's vector at column c covers pairs c/2 .. c/2 + VEC/2 - 1
+    float f[ITER][VEC * 2];
+    if (ROPE) {
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int c = (it * G + lane) * VEC;
+            if (ok) {
+                const float* fp = p.pe + b * p.pe_sb + pos * (2 * D) + c * 2;
+#pragma unroll
+                for (int i = 0; i < VEC * 2 / 4; ++i) {
+                    Vec16<float> t = ld16(fp + i * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) f[it][i * 4 + e] = t.v[e];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < VEC * 2; ++i) f[it][i] = 0.0f;
+            }
+        }
+    }
+
+    // v: bit-exact copy
+    if (p.v.out != nullptr && ok) {
+        bool is_txt;
+        const T* src = src_row<T>(p.v, b, h, pos, p.Lt, is_txt);
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int c = (it * G + lane) * VEC;
+            st16(static_cast<T*>(p.v.out) + out_row + c, ld16(src + c));
+        }
+    }
+
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Src& s = which == 0 ? p.q : p.k;
+        if (s.out == nullptr) continue;  // uniform over the grid
+        T* out = static_cast<T*>(s.out) + out_row;
+        bool is_txt = false;
+        Vec16<T> raw[ITER];
+        if (ok) {
+            const T* src = src_row<T>(s, b, h, pos, p.Lt, is_txt);
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) raw[it] = ld16(src + (it * G + lane) * VEC);
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITER; ++it)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) raw[it].v[e] = T(0);
+        }
+        if (!NORM && !ROPE) {
+            if (ok) {
+#pragma unroll
+                for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, raw[it]);
+            }
+            continue;
+        }
+        float x[ITER][VEC];
+#pragma unroll
+        for (int it = 0; it < ITER; ++it)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[it][e] = Elem<T>::load(raw[it].v[e]);
+        if (NORM) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) ss += x[it][e] * x[it][e];
+            ss = group_sum<G>(ss);  // every lane of the wave takes part, rows past the end hold zeros
+            const float rstd = rsqrtf(ss / static_cast<float>(D) + p.eps);
+            const TS* sc = static_cast<const TS*>(is_txt ? s.scale_txt : s.scale_img);
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int c = (it * G + lane) * VEC;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float w = ok ? Elem<TS>::load(sc[c + e]) : 0.0f;
+                    x[it][e] = Elem<T>::round(Elem<T>::round(x[it][e] * rstd) * w);
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            Vec16<T> o;
+            if (ROPE) {
+#pragma unroll
+                for (int i = 0; i < VEC / 2; ++i) {
+                    const float x0 = x[it][2 * i], x1 = x[it][2 * i + 1];
+                    o.v[2 * i] = Elem<T>::store(f[it][4 * i + 0] * x0 + f[it][4 * i + 1] * x1);
+                    o.v[2 * i + 1] = Elem<T>::store(f[it][4 * i + 2] * x0 + f[it][4 * i + 3] * x1);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o.v[e] = Elem<T>::store(x[it][e]);
+            }
+            if (ok) st16(out + (it * G + lane) * VEC, o);
+        }
+    }
+}
+
+static bool src_ok(const flux_src4& s, int vec) {
+    return s.ptr != nullptr && aligned16(s.ptr) && s.sb % vec == 0 && s.sh % vec == 0 && s.sl % vec == 0;
+}
+
+template <typename T, typename TS>
+static int prep_launch(const flux_qkv_prep_args& a, hipStream_t st) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int64_t L = a.Lt + a.Li;
+    PrepParams p;
+    const flux_src4* txt[3] = {&a.q_txt, &a.k_txt, &a.v_txt};
+    const flux_src4* img[3] = {&a.q_img, &a.k_img, &a.v_img};
+    void* outs[3] = {a.q_out, a.k_out, a.v_out};
+    const void* sc_t[3] = {a.q_scale_txt, a.k_scale_txt, nullptr};
+    const void* sc_i[3] = {a.q_scale_img, a.k_scale_img, nullptr};
+    Src* dst[3] = {&p.q, &p.k, &p.v};
+    const bool norm = a.q_scale_txt || a.q_scale_img || a.k_scale_txt || a.k_scale_img;
+    bool any = false;
+    for (int i = 0; i < 3; ++i) {
+        Src& s = *dst[i];
+        s = Src{};
+        if (outs[i] == nullptr) continue;
+        any = true;
+        if (!aligned16(outs[i])) return fail(FLUX_E_ALIGN, "flux_qkv_prep: output %d is not 16-byte aligned", i);
+        if (a.Lt > 0 && !src_ok(*txt[i], VEC)) return fail(FLUX_E_ALIGN, "flux_qkv_prep: txt source %d is null or not 16-byte addressable", i);
+        if (a.Li > 0 && !src_ok(*img[i], VEC)) return fail(FLUX_E_ALIGN, "flux_qkv_prep: img source %d is null or not 16-byte addressable", i);
+        s.txt = txt[i]->ptr; s.t_sb = txt[i]->sb; s.t_sh = txt[i]->sh; s.t_sl = txt[i]->sl;
+        s.img = img[i]->ptr; s.i_sb = img[i]->sb; s.i_sh = img[i]->sh; s.i_sl = img[i]->sl;
+        s.out = outs[i];
+        if (i < 2 && norm) {
+            if ((a.Lt > 0 && !sc_t[i]) || (a.Li > 0 && !sc_i[i])) return fail(FLUX_E_NULL, "flux_qkv_prep: RMS scale missing for tensor %d", i);
+            s.scale_txt = sc_t[i];
+            s.scale_img = sc_i[i];
+        }
+    }
+    if (!any) return FLUX_OK;
+    const bool rope = a.pe != nullptr;
+    if (rope && !aligned16(a.pe)) return fail(FLUX_E_ALIGN, "flux_qkv_prep: pe is not 16-byte aligned");
+    if (rope && a.pe_batch_stride % 4 != 0) return fail(FLUX_E_ALIGN, "flux_qkv_prep: pe batch stride must be a multiple of 4");
+    p.pe = a.pe;
+    p.pe_sb = a.pe_batch_stride;
+    p.H = a.H; p.Lt = a.Lt; p.L = L; p.eps = a.eps;
+
+    const int D = a.D;
+    const int lanes_per_row = D / VEC < 64 ? D / VEC : 64;
+    const int rows_per_block = kPrepBlock / (lanes_per_row > 0 ? lanes_per_row : 1);
+    dim3 grid((unsigned)((L + rows_per_block - 1) / rows_per_block), (unsigned)(a.B * a.H));
+    if (a.B * a.H > 65535) return fail(FLUX_E_SHAPE, "flux_qkv_prep: B*H = %lld exceeds 65535", (long long)(a.B * a.H));
+
+#define LAUNCH(D_, N_, R_) hipLaunchKernelGGL((qkv_prep_kernel<T, TS, D_, N_, R_>), grid, dim3(kPrepBlock), 0, st, p)
+#define BY_FLAGS(D_)                                   \
+    do {                                               \
+        if (norm && rope) LAUNCH(D_, true, true);      \
+        else if (norm) LAUNCH(D_, true, false);        \
+        else if (rope) LAUNCH(D_, false, true);        \
+        else LAUNCH(D_, false, false);                 \
+    } while (0)
+    if (D == 16) BY_FLAGS(16);
+    else if (D == 32) BY_FLAGS(32);
+    else if (D == 64) BY_FLAGS(64);
+    else if (D == 128) BY_FLAGS(128);
+    else if (D == 256) BY_FLAGS(256);
+    else if (D == 512) BY_FLAGS(512);
+    else return fail(FLUX_E_UNSUPPORTED, "flux_qkv_prep: head dim %d not supported (16, 32, 64, 128, 256, 512)", D);
+#undef BY_FLAGS
+#undef LAUNCH
+    return check_launch("flux_qkv_prep");
+}
+
+}  // namespace flux
+
+using namespace flux;
+
+extern "C" int flux_qkv_prep(const flux_qkv_prep_args* a, void* stream) {
+    if (!a) return fail(FLUX_E_NULL, "flux_qkv_prep: null args");
+    if (a->B < 0 || a->H <= 0 || a->Lt < 0 || a->Li < 0 || a->D <= 0) return fail(FLUX_E_SHAPE, "flux_qkv_prep: bad shape B=%lld H=%lld Lt=%lld Li=%lld D=%d", (long long)a->B, (long long)a->H, (long long)a->Lt, (long long)a->Li, a->D);
+    if (a->B == 0 || a->Lt + a->Li == 0) return FLUX_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (a->dtype == FLUX_BF16 && a->scale_dtype == FLUX_BF16) return prep_launch<bf16_t, bf16_t>(*a, st);
+    if (a->dtype == FLUX_BF16 && a->scale_dtype == FLUX_F32) return prep_launch<bf16_t, float>(*a, st);
+    if (a->dtype == FLUX_F32 && a->scale_dtype == FLUX_F32) return prep_launch<float, float>(*a, st);
+    return fail(FLUX_E_DTYPE, "flux_qkv_prep: unsupported dtype pair (%d,%d)", a->dtype, a->scale_dtype);
+}

@@ -1,0 +1,86 @@
+"""linear: y = act(x @ w.T + b) on the bf16 matrix cores (kernels/linear.py:104-151 of the reference),
+with the extra epilogues the fused Flux blocks use."""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from triton_kernels import _native as nv
+
+_ACTIVATIONS = {"": nv.ACT_NONE, "GELU": nv.ACT_GELU_TANH}
+# Tile plan per dtype; like the reference's table it has a single entry, so any other dtype is a KeyError.
+_PLANS = {torch.bfloat16: {"tile": (256, 256, 64), "waves": 4, "mfma": "32x32x16"}}
+
+
+def _rows_2d(x: Tensor, K: int) -> Tensor:
+    x2 = x.reshape(-1, K)
+    if x2.shape[0] > 1 and (x2.stride(1) != 1 or x2.stride(0) < K):
+        x2 = x2.contiguous()
+    elif x2.shape[0] <= 1 and x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    return x2
+
+
+def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "", act_begin: int = 0,
+                out: Tensor | None = None, out2: Tensor | None = None, split: int | None = None,
+                resid: Tensor | None = None, gate: Tensor | None = None) -> Tensor:
+    """General form of the fused linear.
+
+    out   : [M, >=split] destination (row stride free) for columns [0, split)
+    out2  : destination for columns [split, N), written starting at its column 0
+    act_begin : GELU applies to columns >= act_begin only
+    resid, gate : y = resid + gate * y with resid [..., N] and gate [B, 1, N] (or [B, N])
+    """
+    assert x.shape[-1] == w.shape[-1], "Incompatible dimensions"
+    assert x.dtype == w.dtype, "Incompatible dtypes"
+    _PLANS[x.dtype]  # KeyError for anything but bfloat16, as in the reference
+    act = _ACTIVATIONS[activation]
+    dev = nv.require_gpu(x, w, b, out, out2, resid, gate)
+    N, K = w.shape
+    x2 = _rows_2d(x, K)
+    M = x2.shape[0]
+    if w.stride(1) != 1 or (N > 1 and w.stride(0) < K):
+        w = w.contiguous()
+    if b is not None:
+        assert b.shape[-1] == N
+        b = b.to(x.dtype).contiguous()
+    a = nv.LinearArgs()
+    a.A, a.W, a.bias = x2.data_ptr(), w.data_ptr(), nv.ptr(b)
+    a.M, a.N, a.K = M, N, K
+    a.lda = x2.stride(0) if M > 1 else K
+    a.ldw = w.stride(0) if N > 1 else K
+    if out is None:
+        out = torch.empty((M, N if split is None else split), device=dev, dtype=x.dtype)
+    assert out.dim() == 2 and out.shape[0] == M and out.stride(1) == 1 and out.dtype == x.dtype
+    a.Y, a.ldy = out.data_ptr(), out.stride(0)
+    if split is not None and split < N:
+        assert out2 is not None and out2.dim() == 2 and out2.shape[0] == M and out2.stride(1) == 1
+        assert out.shape[1] >= split and out2.shape[1] >= N - split and out2.dtype == x.dtype
+        a.Y2, a.ldy2, a.split_n, a.y2_col0 = out2.data_ptr(), out2.stride(0), split, 0
+    else:
+        assert out.shape[1] >= N
+        a.Y2, a.split_n = None, N
+    if gate is not None:
+        assert resid is not None
+        r2 = resid.reshape(-1, N)
+        assert r2.shape[0] == M and r2.stride(1) == 1 and r2.dtype == x.dtype
+        g2 = gate.reshape(-1, N) if gate.is_contiguous() else gate.reshape(gate.shape[0], N)
+        if g2.dtype != x.dtype:
+            g2 = g2.to(x.dtype)
+        if g2.stride(1) != 1:
+            g2 = g2.contiguous()
+        nb = g2.shape[0]
+        assert M % nb == 0
+        a.resid, a.ldresid = r2.data_ptr(), r2.stride(0)
+        a.gate, a.gate_batch_stride, a.rows_per_batch = g2.data_ptr(), (g2.stride(0) if nb > 1 else N), M // nb
+    a.act, a.act_begin = act, act_begin
+    with nv.on_device(dev):
+        rc = nv.lib().flux_linear_bf16(nv.byref(a), nv.stream_ptr(dev))
+    nv.check(rc, "flux_linear_bf16")
+    return out
+
+
+def linear(x: Tensor, w: Tensor, b: Tensor | None, activation: str = "") -> Tensor:
+    N = w.shape[0]
+    y = linear_into(x, w, b, activation=activation)
+    return y.reshape(*x.shape[:-1], N)
