@@ -125,9 +125,11 @@ int flux_qkv_prep(const flux_qkv_prep_args* args, void* stream);
  * A is [M,K] with row stride lda, W is [N,K] (nn.Linear layout) with row stride ldw.
  *
  * Epilogue, applied in this order on the fp32 accumulator:
- *   + bias[n] (nullable)                 -> rounded to bf16
- *   tanh-GELU for columns n >= act_begin when act == FLUX_ACT_GELU_TANH (evaluated on the rounded
- *       value, as kernels/linear.py:92-95 does), rounded to bf16
+ *   + bias[n] (nullable)
+ *   tanh-GELU for columns n >= act_begin when act == FLUX_ACT_GELU_TANH, evaluated in fp32 on the
+ *       un-rounded sum (kernels/linear.py:92-95 rounds to bf16 first; one rounding keeps the result
+ *       within half a bf16 ulp of the fp32 value)
+ *   -> rounded to bf16
  *   if gate != null:  y = resid[m,n] + gate[(m / rows_per_batch), n] * y   (each step rounded to
  *       bf16), the gated residual of modules/blocks.py:123
  * Output columns [0, split_n) go to Y (row stride ldy); columns [split_n, N) go to Y2 at column

@@ -13,8 +13,8 @@
 // side stores whole rows, also conflict-free.
 //
 // The MFMA takes W as its "A" operand and the activations as its "B" operand, so the accumulator
-// of a lane holds one activation row m and runs of 4 consecutive output columns n: bias, rounding
-// and GELU are applied there, the bf16 tile goes through LDS once more and leaves as full 16-byte
+// of a lane holds one activation row m and runs of 4 consecutive output columns n: bias and GELU
+// are applied there in fp32 and the result is rounded once, the bf16 tile goes through LDS once more and leaves as full 16-byte
 // row segments, where the optional gated residual is applied.
 #include "common.h"
 #include <stdlib.h>
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float t = bf2f(f2bf(acc[i][j][g * 4 + e] + bv[e]));
+                    float t = acc[i][j][g * 4 + e] + bv[e];
                     if (p.act == FLUX_ACT_GELU_TANH && n + e >= p.act_begin) t = gelu_tanh_f32(t);
                     v[e] = t;
                 }
@@ -308,8 +308,9 @@ __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
     if (lane == 0) {
         const float b = p.bias ? bf2f(p.bias[n]) : 0.0f;
         for (int m = 0; m < p.M && m < MMAX; ++m) {
-            float t = bf2f(f2bf(acc[m] + b));
-            if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = bf2f(f2bf(gelu_tanh_f32(t)));
+            float t = acc[m] + b;
+            if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
+            t = bf2f(f2bf(t));
             if (p.gate != nullptr) {
                 const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
                 const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
@@ -334,8 +335,9 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     const bf16_t* w = p.W + static_cast<int64_t>(n) * p.ldw;
     float acc = 0.0f;
     for (int k = 0; k < p.K; ++k) acc += bf2f(a[k]) * bf2f(w[k]);
-    float t = bf2f(f2bf(acc + (p.bias ? bf2f(p.bias[n]) : 0.0f)));
-    if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = bf2f(f2bf(gelu_tanh_f32(t)));
+    float t = acc + (p.bias ? bf2f(p.bias[n]) : 0.0f);
+    if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
+    t = bf2f(f2bf(t));
     if (p.gate != nullptr) {
         const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
         const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
