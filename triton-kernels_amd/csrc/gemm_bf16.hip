@@ -4,13 +4,14 @@
 // feeds 8 consecutive k of one row. A workgroup of four waves (2 x 2) owns a (64*MI) x (64*NJ) tile
 // of Y and each wave a (32*MI) x (32*NJ) sub-tile kept as MI*NJ accumulators of 32x32. The K loop
 // moves 64-wide slabs of A and W through a two-stage LDS ring: while the MFMAs consume stage s, the
-// slab for the next step lands in stage s^1, either straight from the buffer load (DIRECT) or via
-// registers.
+// slab for the next step lands in stage s^1 straight from buffer loads that write LDS (no register
+// staging).
 //
 // LDS slab layout: row r of the slab is 128 bytes = eight 16-byte chunks; chunk c is stored at
-// position c ^ (r & 7). Eight lanes that read the same logical chunk of eight consecutive rows then
-// touch eight different positions, i.e. all 32 banks once: conflict-free ds_read_b128; the writer
-// side stores whole rows, also conflict-free.
+// position c ^ ((r >> 1) & 7). LDS on gfx950 has 64 banks of 4 bytes, so a ds_read_b128 is served 16
+// lanes (256 bytes) per clock: the 16 lanes that read the same logical chunk of 16 consecutive rows
+// land on 2 (row parity) x 8 (position) = 16 different 16-byte bank groups, conflict-free. The
+// writer side fills whole rows, also conflict-free.
 //
 // The MFMA takes W as its "A" operand and the activations as its "B" operand, so the accumulator
 // of a lane holds one activation row m and runs of 4 consecutive output columns n: bias and GELU
@@ -18,6 +19,7 @@
 // row segments, where the optional gated residual is applied.
 #include "common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace flux {
 
@@ -45,7 +47,6 @@ constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
 constexpr uint32_t kOutOfRange = 0x80000000u;
 
 // LDS-direct buffer loads are counted by vmcnt; the workgroup barrier alone does not wait for them.
-__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 __device__ __forceinline__ u32x2 pack4_bf16(float a, float b, float c, float d) {
     u32x2 r;
@@ -73,27 +74,50 @@ __device__ __forceinline__ bool tile_of_block(const GemmParams& p, int& tm, int&
     return true;
 }
 
-template <int MI, int NJ, bool DIRECT>
+// One buffer load of 64 x 16 bytes, written by the memory pipeline straight into LDS at dst
+// (+ lane * 16, implied by the instruction). `soff` is the scalar byte offset of the slab inside the
+// rows; a vector offset with the top bit set is out of range for the resource and yields zeros.
+__device__ __forceinline__ void load_chunk(__amdgpu_buffer_rsrc_t rsrc, char* dst, uint32_t voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soff, 0, 0);
+}
+
+__device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Which of a slab's LPS buffer loads goes into issue slot g of SLOTS (-1 = none): spread evenly, so
+// the texture-address unit (64 bytes per clock per CU) is never asked for more than it can take and
+// the in-order wave does not stall MFMA issue behind a full memory queue.
+constexpr int load_at_slot(int g, int slots, int lps) {
+    for (int l = 0; l < lps; ++l)
+        if (l * slots / lps == g) return l;
+    return -1;
+}
+
+template <int MI, int NJ>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
-    constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64;
-    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
-    constexpr int PA = BM / 32, PB = BN / 32;  // 32-row passes of the 256-thread loader
+    constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64, NS = 2;
+    constexpr int ROWB = BK * 2;                 // bytes per slab row
+    constexpr int KSUB = BK / 16;                // MFMA K-steps per slab (4)
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int PA = BM / 32, PB = BN / 32;    // loader passes per slab (32 rows = 4096 bytes each)
+    constexpr int LPS = PA + PB;                 // buffer loads per thread per slab
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
     constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;  // epilogue tile: bytes per row, 16-byte chunks per row
-    static_assert(4 * WROWS * C_PITCH <= 2 * STAGE, "epilogue tile must fit the ring");
-    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+    static_assert(4 * WROWS * C_PITCH <= NS * STAGE, "epilogue tile must fit the ring");
+    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
     int tm, tn;
     if (!tile_of_block(p, tm, tn)) return;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases in SGPRs
     const int wm = wave >> 1, wn = wave & 1;
 
-    // ---- loader mapping: thread -> LDS slot (row = pass*32 + tid/8, position tid%8), which holds
-    //      logical chunk (tid%8) ^ (row&7) of that row.
+    // ---- loader mapping: a wave's buffer load drops 64 x 16 bytes into 1 KB of consecutive LDS,
+    //      i.e. thread -> LDS slot (row = pass*32 + tid/8, position tid%8), so the thread fetches
+    //      logical chunk position ^ ((row>>1)&7) of that row from memory.
     const int lrow = tid >> 3;
-    const int lchunk = (tid & 7) ^ (lrow & 7);
+    const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
     const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BN);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda), 0,
@@ -112,55 +136,28 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
         const int r = i * 32 + lrow;
         voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
     }
-    const int lds_slot = lrow * 128 + (tid & 7) * 16;  // within a 32-row pass
 
-    u32x4 stage_a[DIRECT ? 1 : PA], stage_b[DIRECT ? 1 : PB];
-
-    auto issue_loads = [&](int kt, int stage) {
-        const int k0 = kt * BK;
-        const bool kin = k0 + lchunk * 8 < p.K;  // K is a multiple of 8: a chunk is all in or all out
-        const uint32_t kb = static_cast<uint32_t>(k0 * 2);
-        char* sa = lds + stage * STAGE;
-        char* sb = sa + A_BYTES;
-#pragma unroll
-        for (int i = 0; i < PA; ++i) {
-            const uint32_t vo = kin ? voff_a[i] + kb : kOutOfRange;
-            if constexpr (DIRECT) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 4096 + wave * 1024), 16, vo, 0, 0, 0);
-            } else {
-                stage_a[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < PB; ++i) {
-            const uint32_t vo = kin ? voff_b[i] + kb : kOutOfRange;
-            if constexpr (DIRECT) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rsrc_b, (__attribute__((address_space(3))) void*)(sb + i * 4096 + wave * 1024), 16, vo, 0, 0, 0);
-            } else {
-                stage_b[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, 0, 0);
-            }
-        }
+    const int nk = (p.K + BK - 1) / BK;
+    const bool k_ragged = (p.K % BK) != 0;
+    // The part of a slab past K is padded with zeros (K is a multiple of 8, so a 16-byte chunk is all
+    // in or all out).
+    auto slab_kmask = [&](int kt) -> uint32_t {
+        return (k_ragged && kt * BK + lchunk * 8 >= p.K) ? kOutOfRange : 0u;
     };
-    auto commit_loads = [&](int stage) {  // register path only
-        if constexpr (!DIRECT) {
-            char* sa = lds + stage * STAGE;
-            char* sb = sa + A_BYTES;
-#pragma unroll
-            for (int i = 0; i < PA; ++i) *reinterpret_cast<u32x4*>(sa + i * 4096 + lds_slot) = stage_a[i];
-#pragma unroll
-            for (int i = 0; i < PB; ++i) *reinterpret_cast<u32x4*>(sb + i * 4096 + lds_slot) = stage_b[i];
-        }
+    // idx-th of the LPS buffer loads of slab kt: first the PA passes of A, then the PB passes of W
+    auto issue_load = [&](int kt, uint32_t kmask, int idx) {
+        char* sa = lds + (kt & 1) * STAGE + wave * 1024;
+        if (idx < PA) load_chunk(rsrc_a, sa + idx * 4096, voff_a[idx] | kmask, kt * (BK * 2));
+        else load_chunk(rsrc_b, sa + A_BYTES + (idx - PA) * 4096, voff_b[idx - PA] | kmask, kt * (BK * 2));
     };
 
     // ---- fragment addressing
     const int frow = lane & 31, fhalf = lane >> 5;
-    int koff[4];
+    int koff[KSUB];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) koff[kk] = ((kk * 2 + fhalf) ^ (lane & 7)) * 16;
-    const int a_off = (wm * WROWS + frow) * 128;
-    const int b_off = A_BYTES + (wn * WCOLS + frow) * 128;
+    for (int kk = 0; kk < KSUB; ++kk) koff[kk] = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
+    const int a_off = (wm * WROWS + frow) * ROWB;
+    const int b_off = A_BYTES + (wn * WCOLS + frow) * ROWB;
 
     f32x16 acc[MI][NJ];
 #pragma unroll
@@ -170,31 +167,95 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    const int nk = (p.K + BK - 1) / BK;
-    issue_loads(0, 0);
-    commit_loads(0);
-    if constexpr (DIRECT) wait_vmem();
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) issue_loads(kt + 1, cur ^ 1);
-        const char* s = lds + cur * STAGE;
+    bf16x8 xa[2][MI], wb[2][NJ];  // two fragment sets: one feeds the MFMAs while the other is being read
+    auto read_frag = [&](int buf, const char* s, int kk, int r) {
+        // r-th fragment read of a step, in the order the MFMAs (activation block outer, weight
+        // block inner) first need them: x0, w0..w(NJ-1), x1..x(MI-1)
+        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(s + a_off + koff[kk]);
+        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(s + b_off + (r - 1) * 32 * ROWB + koff[kk]);
+        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(s + a_off + (r - NJ) * 32 * ROWB + koff[kk]);
+    };
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / NJ, j = idx % NJ;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
+    };
+    constexpr int READS = MI + NJ, MFMAS = MI * NJ, PER = MFMAS / READS;
+    static_assert(MFMAS % READS == 0, "MFMAs per fragment read");
+    // A slab's loads are issued over three K=16 steps: the step after the barrier that freed the
+    // stage (step 3 of the previous slab) and steps 0 and 1; step 2 stays free so that the loads have
+    // a few hundred cycles to land before the wait in front of the next barrier.
+    constexpr int SLOTS = 3 * READS;
+    // One K=16 step in a fixed interleave: every fragment read of the NEXT step is followed by PER
+    // MFMAs of the current one, so by the time a fragment is needed it was requested a whole step
+    // (>= 256 cycles) earlier; buffer loads of slab `load_kt` are dropped into their issue slots
+    // [slot0, slot0 + READS). The scheduling barriers pin this order; the compiler only adds the
+    // wait counts.
+    auto step = [&](int cur_buf, const char* nxt, int nxt_kk, auto has_next, auto slot0, int load_kt, uint32_t load_kmask) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            bf16x8 xa[MI], wb[NJ];
+        for (int r = 0; r < READS; ++r) {
+            if constexpr (decltype(has_next)::value) read_frag(cur_buf ^ 1, nxt, nxt_kk, r);
+            constexpr int S0 = decltype(slot0)::value;
+            if constexpr (S0 >= 0) {
+                const int l = load_at_slot(S0 + r, SLOTS, LPS);
+                if (l >= 0) issue_load(load_kt, load_kmask, l);
+            }
 #pragma unroll
-            for (int i = 0; i < MI; ++i) xa[i] = *reinterpret_cast<const bf16x8*>(s + a_off + i * 4096 + koff[kk]);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) wb[j] = *reinterpret_cast<const bf16x8*>(s + b_off + j * 4096 + koff[kk]);
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[j], xa[i], acc[i][j], 0, 0, 0);
+            for (int m = 0; m < PER; ++m) mfma_one(cur_buf, r * PER + m);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (kt + 1 < nk) commit_loads(cur ^ 1);
-        if constexpr (DIRECT) wait_vmem();
+    };
+    using no_loads = std::integral_constant<int, -1>;
+    // One slab with a successor. `more` says whether a slab kt+2 exists, whose first loads go out in
+    // the step after the barrier.
+    auto slab = [&](int kt, auto more) {
+        const char* s = lds + (kt & 1) * STAGE;
+        const char* sn = lds + ((kt & 1) ^ 1) * STAGE;
+        const uint32_t kmask1 = slab_kmask(kt + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        step(0, s, 1, std::true_type{}, std::integral_constant<int, READS>{}, kt + 1, kmask1);
+        step(1, s, 2, std::true_type{}, std::integral_constant<int, 2 * READS>{}, kt + 1, kmask1);
+        step(0, s, 3, std::true_type{}, no_loads{}, 0, 0u);
+        wait_vmem_all();   // this wave's share of slab kt+1 has landed ...
+        __syncthreads();   // ... and so has everybody else's; all waves are done reading slab kt-1's stage
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (decltype(more)::value)
+            step(1, sn, 0, std::true_type{}, std::integral_constant<int, 0>{}, kt + 2, slab_kmask(kt + 2));
+        else
+            step(1, sn, 0, std::true_type{}, no_loads{}, 0, 0u);
+    };
+
+    // Prologue: slab 0 completely, then the first third of slab 1.
+    {
+        const uint32_t km = slab_kmask(0);
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) issue_load(0, km, i);
+        wait_vmem_all();
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
+        if (nk > 1) {
+            const uint32_t km1 = slab_kmask(1);
+#pragma unroll
+            for (int g = 0; g < READS; ++g) {
+                const int l = load_at_slot(g, SLOTS, LPS);
+                if (l >= 0) issue_load(1, km1, l);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) slab(kt, std::true_type{});
+    if (kt + 1 < nk) {
+        slab(kt, std::false_type{});
+        ++kt;
+    }
+    {
+        const char* s = lds + (kt & 1) * STAGE;
+        step(0, s, 1, std::true_type{}, no_loads{}, 0, 0u);
+        step(1, s, 2, std::true_type{}, no_loads{}, 0, 0u);
+        step(0, s, 3, std::true_type{}, no_loads{}, 0, 0u);
+        step(1, nullptr, 0, std::false_type{}, no_loads{}, 0, 0u);
         __syncthreads();
     }
 
@@ -348,7 +409,7 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     *dst = f2bf(t);
 }
 
-template <int MI, int NJ, bool DIRECT>
+template <int MI, int NJ>
 static void launch_tiled(GemmParams& p, hipStream_t st) {
     constexpr int BM = 64 * MI, BN = 64 * NJ;
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -356,7 +417,7 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     p.group_m = 4;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ, DIRECT>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
 // Selected by FLUX_GEMM_VARIANT for experiments: 0 = automatic.
@@ -420,11 +481,9 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     }
     const int variant = gemm_variant();
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-    if (variant == 1) launch_tiled<4, 4, false>(p, st);
-    else if (variant == 2) launch_tiled<4, 4, true>(p, st);
-    else if (variant == 3) launch_tiled<2, 2, false>(p, st);
-    else if (variant == 4) launch_tiled<2, 2, true>(p, st);
-    else if (big_tiles >= 192) launch_tiled<4, 4, false>(p, st);
-    else launch_tiled<2, 2, false>(p, st);
+    if (variant == 1) launch_tiled<4, 4>(p, st);
+    else if (variant == 2) launch_tiled<2, 2>(p, st);
+    else if (big_tiles >= 192) launch_tiled<4, 4>(p, st);
+    else launch_tiled<2, 2>(p, st);
     return check_launch("flux_linear_bf16");
 }
