@@ -81,6 +81,10 @@ __device__ __forceinline__ void load_chunk(__amdgpu_buffer_rsrc_t rsrc, char* ds
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soff, 0, 0);
 }
 
+__device__ __forceinline__ u32x4 load_chunk_reg(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+}
+
 __device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Which of a slab's LPS buffer loads goes into issue slot g of SLOTS (-1 = none): spread evenly, so
@@ -92,7 +96,7 @@ constexpr int load_at_slot(int g, int slots, int lps) {
     return -1;
 }
 
-template <int MI, int NJ>
+template <int MI, int NJ, bool STAGED>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
     constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64, NS = 2;
     constexpr int ROWB = BK * 2;                 // bytes per slab row
@@ -143,6 +147,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
     // in or all out).
     auto slab_kmask = [&](int kt) -> uint32_t {
         return (k_ragged && kt * BK + lchunk * 8 >= p.K) ? kOutOfRange : 0u;
+    };
+    // Register-staged path: slab data waits in registers (one 16-byte chunk per load) until its ring
+    // stage is free, which takes the memory pipeline off the critical path: a load issued in slot g
+    // is not needed before slot g of the next slab.
+    u32x4 sreg[STAGED ? LPS : 1];
+    const int lds_slot = lrow * 128 + (tid & 7) * 16;  // within a 32-row pass
+    auto stage_load = [&](int kt, int idx) {   // global -> sreg[idx]; slabs past the end read as zeros
+        const uint32_t kmask = (kt >= nk || (k_ragged && kt * BK + lchunk * 8 >= p.K)) ? kOutOfRange : 0u;
+        if (idx < PA) sreg[idx] = load_chunk_reg(rsrc_a, voff_a[idx] | kmask, kt * (BK * 2));
+        else sreg[idx] = load_chunk_reg(rsrc_b, voff_b[idx - PA] | kmask, kt * (BK * 2));
+    };
+    auto stage_store = [&](int kt, int idx) {  // sreg[idx] -> ring stage of slab kt
+        char* sa = lds + (kt & 1) * STAGE + lds_slot;
+        if (idx < PA) *reinterpret_cast<u32x4*>(sa + idx * 4096) = sreg[idx];
+        else *reinterpret_cast<u32x4*>(sa + A_BYTES + (idx - PA) * 4096) = sreg[idx];
     };
     // idx-th of the LPS buffer loads of slab kt: first the PA passes of A, then the PB passes of W
     auto issue_load = [&](int kt, uint32_t kmask, int idx) {
@@ -195,9 +214,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
         for (int r = 0; r < READS; ++r) {
             if constexpr (decltype(has_next)::value) read_frag(cur_buf ^ 1, nxt, nxt_kk, r);
             constexpr int S0 = decltype(slot0)::value;
-            if constexpr (S0 >= 0) {
+            if constexpr (S0 >= 0 && !STAGED) {
                 const int l = load_at_slot(S0 + r, SLOTS, LPS);
                 if (l >= 0) issue_load(load_kt, load_kmask, l);
+            }
+            if constexpr (S0 >= 0 && STAGED) {
+                // load_kt = the slab whose chunk goes from registers to LDS in this slot; the freed
+                // register is refilled with the same chunk of the slab after it
+                const int l = load_at_slot(S0 + r, 4 * READS, LPS);
+                if (l >= 0) {
+                    stage_store(load_kt, l);
+                    stage_load(load_kt + 1, l);
+                }
             }
 #pragma unroll
             for (int m = 0; m < PER; ++m) mfma_one(cur_buf, r * PER + m);
@@ -210,8 +238,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
     auto slab = [&](int kt, auto more) {
         const char* s = lds + (kt & 1) * STAGE;
         const char* sn = lds + ((kt & 1) ^ 1) * STAGE;
-        const uint32_t kmask1 = slab_kmask(kt + 1);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (STAGED) {
+            // slots 8..31 move chunks of slab kt+1 into the other stage, the barrier publishes them
+            // and frees this slab's stage, whose first chunks (slab kt+2) follow in slots 0..7
+            step(0, s, 1, std::true_type{}, std::integral_constant<int, READS>{}, kt + 1, 0u);
+            step(1, s, 2, std::true_type{}, std::integral_constant<int, 2 * READS>{}, kt + 1, 0u);
+            step(0, s, 3, std::true_type{}, std::integral_constant<int, 3 * READS>{}, kt + 1, 0u);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            step(1, sn, 0, std::true_type{}, std::integral_constant<int, 0>{}, kt + 2, 0u);
+            return;
+        }
+        const uint32_t kmask1 = slab_kmask(kt + 1);
         step(0, s, 1, std::true_type{}, std::integral_constant<int, READS>{}, kt + 1, kmask1);
         step(1, s, 2, std::true_type{}, std::integral_constant<int, 2 * READS>{}, kt + 1, kmask1);
         step(0, s, 3, std::true_type{}, no_loads{}, 0, 0u);
@@ -224,8 +263,29 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
             step(1, sn, 0, std::true_type{}, no_loads{}, 0, 0u);
     };
 
+    if constexpr (STAGED) {
+        // Prologue: slab 0 through the registers into stage 0; slab 1 into the registers, and its
+        // chunks that belong to slots 0..7 already into stage 1.
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) stage_load(0, i);
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) stage_store(0, i);
+#pragma unroll
+        for (int i = 0; i < LPS; ++i) stage_load(1, i);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
+#pragma unroll
+        for (int g = 0; g < READS; ++g) {
+            const int l = load_at_slot(g, 4 * READS, LPS);
+            if (l >= 0) {
+                stage_store(1, l);
+                stage_load(2, l);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    } else {
     // Prologue: slab 0 completely, then the first third of slab 1.
-    {
         const uint32_t km = slab_kmask(0);
 #pragma unroll
         for (int i = 0; i < LPS; ++i) issue_load(0, km, i);
@@ -409,7 +469,7 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     *dst = f2bf(t);
 }
 
-template <int MI, int NJ>
+template <int MI, int NJ, bool STAGED>
 static void launch_tiled(GemmParams& p, hipStream_t st) {
     constexpr int BM = 64 * MI, BN = 64 * NJ;
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -417,7 +477,7 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     p.group_m = 4;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ, STAGED>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
 // Selected by FLUX_GEMM_VARIANT for experiments: 0 = automatic.
@@ -481,9 +541,11 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     }
     const int variant = gemm_variant();
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-    if (variant == 1) launch_tiled<4, 4>(p, st);
-    else if (variant == 2) launch_tiled<2, 2>(p, st);
-    else if (big_tiles >= 192) launch_tiled<4, 4>(p, st);
-    else launch_tiled<2, 2>(p, st);
+    if (variant == 1) launch_tiled<4, 4, false>(p, st);
+    else if (variant == 2) launch_tiled<2, 2, false>(p, st);
+    else if (variant == 3) launch_tiled<4, 4, true>(p, st);
+    else if (variant == 4) launch_tiled<2, 2, true>(p, st);
+    else if (big_tiles >= 192) launch_tiled<4, 4, false>(p, st);
+    else launch_tiled<2, 2, false>(p, st);
     return check_launch("flux_linear_bf16");
 }
