@@ -1,0 +1,78 @@
+"""The C-ABI shared library: it loads, exports every symbol include/flux_hip.h declares, the ctypes
+structures have the sizes the header's structs have, and argument checks reject bad input before
+any launch (no GPU needed for any of this)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from triton_kernels import _native as nv
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flux_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flux_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built():
+    assert os.path.exists(nv.lib_path()), "run `python __graft_entry__.py build` first"
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_functions()
+    assert len(names) >= 12
+    handle = ctypes.CDLL(nv.lib_path())
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared in flux_hip.h but not exported"
+    assert set(names) == set(nv.SIGNATURES), "ctypes binding table and header disagree"
+    assert nv.lib().flux_abi_version() == 1
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    src = tmp_path / "sizes.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "flux_hip.h"\n'
+        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu %zu\\n\", sizeof(flux_src4), sizeof(flux_qkv_prep_args), "
+        "sizeof(flux_linear_args), sizeof(flux_attn_args), offsetof(flux_qkv_prep_args, pe), "
+        "offsetof(flux_linear_args, act_begin), offsetof(flux_attn_args, sm_scale));return 0;}\n")
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = [int(t) for t in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    want = [ctypes.sizeof(nv.Src4), ctypes.sizeof(nv.QkvPrepArgs), ctypes.sizeof(nv.LinearArgs), ctypes.sizeof(nv.AttnArgs),
+            nv.QkvPrepArgs.pe.offset, nv.LinearArgs.act_begin.offset, nv.AttnArgs.sm_scale.offset]
+    assert got == want
+
+
+def test_argument_checks_reject_before_launch():
+    lib = nv.lib()
+    assert lib.flux_rms_norm(None, None, None, None, 1, 1, 1, 8, 0, 0, 0, 0, 0, 1e-6, None) == -1      # null pointer
+    assert b"null" in lib.flux_last_error()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    assert lib.flux_rms_norm(p, p, p, None, 1, 1, 1, 70000, 0, 0, 0, 0, 0, 1e-6, None) == -5            # too wide
+    assert b"65536" in lib.flux_last_error()
+    assert lib.flux_rms_norm(p, p, p, None, 1, 1, 1, 8, 0, 0, 0, 7, 0, 1e-6, None) == -3                # dtype
+    assert lib.flux_rms_norm(p, p, p, None, 0, 1, 1, 8, 0, 0, 0, 0, 0, 1e-6, None) == 0                 # empty: no launch
+    assert lib.flux_layer_norm_modulation(p, p, p, p, 1, 1, -2, 8, 0, 1e-6, None) == -2                 # shape
+    a = nv.AttnArgs()
+    a.B, a.H, a.L, a.D = 1, 1, 8, 48
+    assert lib.flux_attention_fwd_bf16(ctypes.byref(a), None) == -6                                     # head dim
+    la = nv.LinearArgs()
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == -1
+    la.A = la.W = la.Y = p
+    la.M, la.N, la.K, la.lda, la.ldw = 4, 4, 16, 8, 16
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == -2                                           # lda < K
+    la.lda, la.act = 16, 9
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == -6                                           # activation
+    la.act, la.M = 0, 0
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == 0                                            # empty
+    assert lib.flux_silu(p, p, -1, 0, None) == -2
+    qa = nv.QkvPrepArgs()
+    qa.B, qa.H, qa.Lt, qa.Li, qa.D = 1, 0, 0, 4, 128
+    assert lib.flux_qkv_prep(ctypes.byref(qa), None) == -2
