@@ -8,11 +8,14 @@
 // the running max / sum / rescale of the online softmax are per-lane scalars; the only cross-lane
 // step is one exchange between the two half-waves that share a query row. P never touches LDS: the
 // 8 accumulator values a lane holds for a 16-key step are exactly the 8 contraction elements the
-// "B" operand wants, provided V^T is laid out with the same key order, which the V loader does.
+// "B" operand wants, provided the V^T fragment uses the same key order, which its two transposing
+// reads (keys 4h..4h+3 and 8+4h..8+4h+3 of the step) do.
 //
-// A workgroup of 4 waves handles 128*QB query rows of one (batch, head); each wave 32*QB rows.
-// K and V tiles of 64 keys are double-buffered in LDS; V is transposed on the way in (4 keys x 8 d
-// per thread, written as eight 8-byte rows of V^T).
+// A workgroup of 4 waves handles 128*QB query rows of one (batch, head); each wave 32*QB rows. With
+// QB = 1 two workgroups share a CU, so each SIMD interleaves two waves and the softmax VALU work of
+// one overlaps the MFMAs of the other. K and V tiles of 64 keys are double-buffered in LDS, both
+// row-major, filled by buffer loads that write LDS directly; the V^T fragments are produced by the
+// transposing LDS read ds_read_b64_tr_b16.
 #include "common.h"
 #include <stdlib.h>
 
@@ -22,6 +25,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 struct AttnParams {
     const bf16_t* q; const bf16_t* k; const bf16_t* v; bf16_t* o; float* lse;
@@ -37,17 +41,30 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
     return static_cast<uint32_t>(f2bf(a)) | (static_cast<uint32_t>(f2bf(b)) << 16);
 }
 
+// One buffer load of 64 x 16 bytes written straight into LDS at dst + lane * 16.
+__device__ __forceinline__ void lds_load16(__amdgpu_buffer_rsrc_t rsrc, char* dst, uint32_t voff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, 0, 0, 0);
+}
+__device__ __forceinline__ void wait_all_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+// ds_read_b64_tr_b16: inside each group of 16 lanes, lanes 4r..4r+3 together supply row r (16
+// consecutive 16-bit elements, 8 bytes per lane) of a 4 x 16 matrix; lane i of the group receives
+// column i, i.e. the 4 elements (row 0..3)[i].
+__device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+}
+
 template <int D, int QB>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnParams p) {
     constexpr int BN = 64;              // keys per tile
     constexpr int KSTEPS = D / 16;      // contraction steps of S^T = K Q^T
     constexpr int DB = D / 32;          // 32-row blocks of O^T
-    constexpr int CH = D / 8;           // 16-byte chunks per K row
-    constexpr int KROW = D * 2;         // bytes per K row in LDS
-    constexpr int K_BYTES = BN * KROW, V_BYTES = D * 128, STAGE = K_BYTES + V_BYTES;
-    constexpr int KPASS = BN * CH / 256;  // K loader passes (16-byte chunks per thread)
-    constexpr int KROWS_PER_PASS = 256 / CH;
-    constexpr int VTHREADS = CH * 16;   // threads that take part in the V loader (4 keys x 8 d each)
+    constexpr int CH = D / 8;           // 16-byte chunks per K / V row
+    constexpr int ROWB = D * 2;         // bytes per K / V row in LDS
+    constexpr int RPW = 64 / CH;        // rows one wave-wide load covers (1 KB)
+    constexpr int PASSES = BN / (4 * RPW);  // loads per thread per operand per tile
+    constexpr int T_BYTES = BN * ROWB, STAGE = 2 * T_BYTES;
     __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
 
     // XCD-aware order: workgroup w runs on XCD w % 8; each XCD gets a contiguous run of
@@ -58,12 +75,19 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     const int bh = vt / p.n_qtiles, qt = vt % p.n_qtiles;
     const int b = bh / p.H, h = bh % p.H;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 31, fhalf = lane >> 5;
     const int q0 = qt * (128 * QB) + wave * (32 * QB);
 
     const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
     const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
+
+    // LDS row swizzles (64 banks of 4 bytes; a b128 read is served 16 lanes per clock, a b64 read 32):
+    //   K rows are read whole-chunk by 16 lanes on 16 consecutive rows  -> chunk ^ kswz(row)
+    //   V rows are read transposed, 4 rows x 64 bytes per clock         -> chunk ^ vswz(row)
+    auto kswz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto vswz = [](int row) { return D == 128 ? ((row & 3) * 4) : (((row >> 1) & 1) * 4); };
 
     // ---- Q fragments ("B" operand): lane holds row q0 + qb*32 + frow, d = (kk*2 + fhalf)*8 .. +8
     bf16x8 qf[QB][KSTEPS];
@@ -83,13 +107,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         }
     }
 
-    // ---- loader mappings
-    const int kl_c = tid % CH, kl_r = tid / CH;             // K: chunk, row within pass
-    const int vl_dc = tid % CH, vl_kg = (tid / CH) & 15;    // V: d-chunk, group of 4 keys
-    const bool v_active = tid < VTHREADS;
-    u32x4 kreg[KPASS], vreg[4];
-
-    auto issue_loads = [&](int key0) {
+    // ---- loader: thread -> LDS slot (row = pass*4*RPW + wave*RPW + lane/CH, position lane%CH)
+    const int l_row = lane / CH, l_pos = lane % CH;
+    auto issue_loads = [&](int key0, int stage) {
         const int rows = min(p.L - key0, BN);
         const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<bf16_t*>(kbase + static_cast<int64_t>(key0) * p.k_sl), 0,
@@ -97,55 +117,31 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<bf16_t*>(vbase + static_cast<int64_t>(key0) * p.v_sl), 0,
             static_cast<int>(((rows - 1) * p.v_sl + D) * 2), kAttnRsrcFlags);
+        char* sk = lds + stage * STAGE + wave * 1024;
+        char* sv = sk + T_BYTES;
 #pragma unroll
-        for (int i = 0; i < KPASS; ++i) {
-            const int r = i * KROWS_PER_PASS + kl_r;
-            const uint32_t vo = r < rows ? static_cast<uint32_t>((r * p.k_sl + kl_c * 8) * 2) : kAttnOutOfRange;
-            kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, vo, 0, 0);
-        }
-        if (v_active) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int r = vl_kg * 4 + i;
-                const uint32_t vo = r < rows ? static_cast<uint32_t>((r * p.v_sl + vl_dc * 8) * 2) : kAttnOutOfRange;
-                vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rv, vo, 0, 0);
-            }
+        for (int i = 0; i < PASSES; ++i) {
+            const int r = i * 4 * RPW + wave * RPW + l_row;
+            const uint32_t ko = r < rows ? static_cast<uint32_t>((r * p.k_sl + (l_pos ^ kswz(r)) * 8) * 2) : kAttnOutOfRange;
+            const uint32_t vo = r < rows ? static_cast<uint32_t>((r * p.v_sl + (l_pos ^ vswz(r)) * 8) * 2) : kAttnOutOfRange;
+            lds_load16(rk, sk + i * 4096, ko);
+            lds_load16(rv, sv + i * 4096, vo);
         }
     };
-    auto commit_loads = [&](int stage) {
-        char* sk = lds + stage * STAGE;
-        char* sv = sk + K_BYTES;
+
+    // ---- fragment addressing
+    // K ("A" of S^T): row kb*32 + frow, chunk kk*2 + fhalf
+    int k_off[2];
 #pragma unroll
-        for (int i = 0; i < KPASS; ++i) {
-            const int r = i * KROWS_PER_PASS + kl_r;
-            *reinterpret_cast<u32x4*>(sk + r * KROW + ((kl_c ^ (r & 7)) * 16)) = kreg[i];
-        }
-        if (v_active) {
-            // vreg[i] = V[key 4*kg + i][d = dc*8 .. +8]; emit for each d one 8-byte run of the 4 keys.
-            // Key order inside a group of 16 is quads [0,2,1,3]: half-wave h of the MFMA then finds its
-            // 8 keys {4h..4h+3, 8+4h..8+4h+3} in one 16-byte unit.
-            const int quad = vl_kg & 3;
-            const int qpos = (quad == 1) ? 2 : (quad == 2 ? 1 : quad);
-            const int u8 = (vl_kg >> 2) * 4 + qpos;  // 8-byte unit inside the 128-byte V^T row
-            const int unit = u8 >> 1, half = u8 & 1;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int d = vl_dc * 8 + e;
-                const int w = e >> 1;
-                uint32_t a0 = vreg[0][w], a1 = vreg[1][w], a2 = vreg[2][w], a3 = vreg[3][w];
-                u32x2 out;
-                if (e & 1) {
-                    out.x = (a0 >> 16) | (a1 & 0xffff0000u);
-                    out.y = (a2 >> 16) | (a3 & 0xffff0000u);
-                } else {
-                    out.x = (a0 & 0xffffu) | (a1 << 16);
-                    out.y = (a2 & 0xffffu) | (a3 << 16);
-                }
-                const int swz = (d & 7) ^ ((d >> 3) & 7);
-                *reinterpret_cast<u32x2*>(sv + d * 128 + ((unit ^ swz) * 16) + half * 8) = out;
-            }
-        }
-    };
+    for (int kb = 0; kb < 2; ++kb) k_off[kb] = (kb * 32 + frow) * ROWB;
+    const int k_sw = kswz(frow);  // kb*32 does not change the swizzle
+    // V^T ("A" of O^T): lane group g = lane/16 -> (half h = g/2 = fhalf, d sub-block g%2); lane j = lane%16
+    // supplies 8 bytes of key row 4h + j/4 (+8 for the second read) at d = db*32 + (g%2)*16 + 4*(j%4)
+    const int vj = lane & 15, vg = (lane >> 4) & 1;
+    const int v_key = 4 * fhalf + (vj >> 2);                  // + 16*ks (+8)
+    const int v_chunk = vg * 2 + ((vj & 3) >> 1);             // + db*4
+    const int v_in = (vj & 1) * 8;
+    const int v_sw = vswz(v_key);                             // unchanged by + 8, + 16*ks
 
     // ---- softmax state (per lane = per query row of each q-block)
     float m_run[QB], l_run[QB];
@@ -162,16 +158,16 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     const float c = p.scale_log2;
 
     const int ntiles = (p.L + BN - 1) / BN;
-    issue_loads(0);
-    commit_loads(0);
+    issue_loads(0, 0);
+    wait_all_vmem();
     __syncthreads();
 
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
         const int key0 = t * BN;
-        if (t + 1 < ntiles) issue_loads(key0 + BN);
+        if (t + 1 < ntiles) issue_loads(key0 + BN, cur ^ 1);
         const char* sk = lds + cur * STAGE;
-        const char* sv = sk + K_BYTES;
+        const char* sv = sk + T_BYTES;
 
         // S^T = K Q^T
         f32x16 s[QB][2];
@@ -185,10 +181,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         for (int kk = 0; kk < KSTEPS; ++kk) {
             bf16x8 kf[2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const int row = kb * 32 + frow;
-                kf[kb] = *reinterpret_cast<const bf16x8*>(sk + row * KROW + (((kk * 2 + fhalf) ^ (lane & 7)) * 16));
-            }
+            for (int kb = 0; kb < 2; ++kb)
+                kf[kb] = *reinterpret_cast<const bf16x8*>(sk + k_off[kb] + (((kk * 2 + fhalf) ^ k_sw) * 16));
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
@@ -213,58 +207,64 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
         bf16x8 pf[QB][4];
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-            float mx = s[qb][0][0];
+            float mx = fmaxf(s[qb][0][0], s[qb][1][0]);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[qb][kb][r]);
+            for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, s[qb][0][r]), s[qb][1][r]);  // v_max3_f32
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run[qb], mx);
-            const float alpha = m_run[qb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c);
+            // The accumulator only needs rescaling when some row's running max moved; after the first
+            // few tiles that is rare, so the whole wave skips the multiplies when no lane needs them.
+            if (__builtin_amdgcn_ballot_w64(m_new != m_run[qb]) != 0) {
+                const float alpha = m_run[qb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c);
+                l_run[qb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[qb][db][r] *= alpha;
+                m_run[qb] = m_new;
+            }
             const float mc = m_new * c;
-            m_run[qb] = m_new;
             float sum = 0.0f;
+            const uint32_t ones = 0x3f803f80u;  // (1.0bf16, 1.0bf16)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                float pv[16];
+                uint32_t w[8];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    pv[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kb][r], c, -mc));
-                    sum += pv[r];
+                for (int r = 0; r < 8; ++r) {
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kb][2 * r], c, -mc));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kb][2 * r + 1], c, -mc));
+                    w[r] = pack2_bf16(p0, p1);
+                    // row sum from the rounded values, two per instruction: sum += p0*1 + p1*1
+                    sum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w[r]), __builtin_bit_cast(bf16x2, ones), sum, false);
                 }
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
-                    u32x4 w;
-                    w.x = pack2_bf16(pv[8 * tt + 0], pv[8 * tt + 1]);
-                    w.y = pack2_bf16(pv[8 * tt + 2], pv[8 * tt + 3]);
-                    w.z = pack2_bf16(pv[8 * tt + 4], pv[8 * tt + 5]);
-                    w.w = pack2_bf16(pv[8 * tt + 6], pv[8 * tt + 7]);
-                    pf[qb][kb * 2 + tt] = __builtin_bit_cast(bf16x8, w);
+                    u32x4 v4 = {w[4 * tt], w[4 * tt + 1], w[4 * tt + 2], w[4 * tt + 3]};
+                    pf[qb][kb * 2 + tt] = __builtin_bit_cast(bf16x8, v4);
                 }
             }
-            l_run[qb] = l_run[qb] * alpha + sum;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[qb][db][r] *= alpha;
+            l_run[qb] += sum;
         }
 
-        // O^T += V^T P^T
+        // O^T += V^T P^T ; V^T fragments come out of row-major V through transposing LDS reads
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const int d = db * 32 + frow;
-                const int swz = (d & 7) ^ ((d >> 3) & 7);
-                const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sv + d * 128 + (((ks * 2 + fhalf) ^ swz) * 16));
+                const char* vp = sv + (ks * 16 + v_key) * ROWB + (((db * 4 + v_chunk) ^ v_sw) * 16) + v_in;
+                const s16x4 lo = lds_read_tr(vp);
+                const s16x4 hi = lds_read_tr(vp + 8 * ROWB);
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb)
                     acc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][ks], acc[qb][db], 0, 0, 0);
             }
         }
 
-        if (t + 1 < ntiles) commit_loads(cur ^ 1);
-        __syncthreads();
+        wait_all_vmem();   // this wave's part of the next tile has landed
+        __syncthreads();   // everybody's has; and everybody is done reading this tile
     }
 
     // ---- finish: fold the two half-waves' partial sums, normalise, store
@@ -339,10 +339,10 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     const int64_t BH = a->B * a->H;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int variant = attn_variant();
-    // Two q-blocks per wave halve the LDS traffic per flop; one q-block gives twice the workgroups,
-    // which small problems need to fill the chip.
-    const bool small = ((a->L + 255) / 256) * BH < 256;
-    const int qb = variant == 1 ? 1 : (variant == 2 ? 2 : (small ? 1 : 2));
+    // One q-block (32 rows) per wave keeps the kernel under 256 registers, so two workgroups share a
+    // CU and the two waves on each SIMD overlap softmax with MFMA; two q-blocks per wave halve the LDS
+    // traffic per flop but run one wave per SIMD.
+    const int qb = variant == 2 ? 2 : 1;
     if (a->D == 128) {
         if (qb == 1) attn_launch<128, 1>(p, BH, st); else attn_launch<128, 2>(p, BH, st);
     } else {
