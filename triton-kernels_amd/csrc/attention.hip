@@ -37,8 +37,12 @@ struct AttnParams {
 constexpr unsigned kAttnRsrcFlags = 0x00020000u;
 constexpr uint32_t kAttnOutOfRange = 0x80000000u;
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// Two floats -> one dword of two bf16 (a in the low half): a single v_cvt_pk_bf16_f32.
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
-    return static_cast<uint32_t>(f2bf(a)) | (static_cast<uint32_t>(f2bf(b)) << 16);
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // One buffer load of 64 x 16 bytes written straight into LDS at dst + lane * 16.
@@ -109,6 +113,15 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
 
     // ---- loader: thread -> LDS slot (row = pass*4*RPW + wave*RPW + lane/CH, position lane%CH)
     const int l_row = lane / CH, l_pos = lane % CH;
+    // Byte offsets of this thread's chunks inside a tile; rows past the end of the sequence fall
+    // outside the buffer resource built for the tile and read as zeros.
+    uint32_t k_voff[PASSES], v_voff[PASSES];
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+        const int r = i * 4 * RPW + wave * RPW + l_row;
+        k_voff[i] = static_cast<uint32_t>((r * p.k_sl + (l_pos ^ kswz(r)) * 8) * 2);
+        v_voff[i] = static_cast<uint32_t>((r * p.v_sl + (l_pos ^ vswz(r)) * 8) * 2);
+    }
     auto issue_loads = [&](int key0, int stage) {
         const int rows = min(p.L - key0, BN);
         const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
@@ -121,19 +134,13 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
         char* sv = sk + T_BYTES;
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) {
-            const int r = i * 4 * RPW + wave * RPW + l_row;
-            const uint32_t ko = r < rows ? static_cast<uint32_t>((r * p.k_sl + (l_pos ^ kswz(r)) * 8) * 2) : kAttnOutOfRange;
-            const uint32_t vo = r < rows ? static_cast<uint32_t>((r * p.v_sl + (l_pos ^ vswz(r)) * 8) * 2) : kAttnOutOfRange;
-            lds_load16(rk, sk + i * 4096, ko);
-            lds_load16(rv, sv + i * 4096, vo);
+            lds_load16(rk, sk + i * 4096, k_voff[i]);
+            lds_load16(rv, sv + i * 4096, v_voff[i]);
         }
     };
 
     // ---- fragment addressing
     // K ("A" of S^T): row kb*32 + frow, chunk kk*2 + fhalf
-    int k_off[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) k_off[kb] = (kb * 32 + frow) * ROWB;
     const int k_sw = kswz(frow);  // kb*32 does not change the swizzle
     // V^T ("A" of O^T): lane group g = lane/16 -> (half h = g/2 = fhalf, d sub-block g%2); lane j = lane%16
     // supplies 8 bytes of key row 4h + j/4 (+8 for the second read) at d = db*32 + (g%2)*16 + 4*(j%4)
@@ -142,6 +149,11 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
     const int v_chunk = vg * 2 + ((vj & 3) >> 1);             // + db*4
     const int v_in = (vj & 1) * 8;
     const int v_sw = vswz(v_key);                             // unchanged by + 8, + 16*ks
+    int k_addr[KSTEPS], v_addr[DB];                           // per-lane parts, the rest are immediates
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) k_addr[kk] = frow * ROWB + (((kk * 2 + fhalf) ^ k_sw) * 16);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) v_addr[db] = T_BYTES + v_key * ROWB + (((db * 4 + v_chunk) ^ v_sw) * 16) + v_in;
 
     // ---- softmax state (per lane = per query row of each q-block)
     float m_run[QB], l_run[QB];
@@ -167,28 +179,25 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
         const int key0 = t * BN;
         if (t + 1 < ntiles) issue_loads(key0 + BN, cur ^ 1);
         const char* sk = lds + cur * STAGE;
-        const char* sv = sk + T_BYTES;
 
         // S^T = K Q^T
         f32x16 s[QB][2];
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[qb][kb][r] = 0.0f;
+        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_setprio(1);  // the other wave on this SIMD is in its softmax: let the MFMAs go first
 #pragma unroll
         for (int kk = 0; kk < KSTEPS; ++kk) {
             bf16x8 kf[2];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-                kf[kb] = *reinterpret_cast<const bf16x8*>(sk + k_off[kb] + (((kk * 2 + fhalf) ^ k_sw) * 16));
+                kf[kb] = *reinterpret_cast<const bf16x8*>(sk + kb * 32 * ROWB + k_addr[kk]);
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
-                    s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[qb][kk], s[qb][kb], 0, 0, 0);
+                    s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[qb][kk], kk == 0 ? zero16 : s[qb][kb], 0, 0, 0);
         }
+
+        __builtin_amdgcn_s_setprio(0);
 
         // ragged tail: keys past L get -inf
         if (key0 + BN > p.L) {
@@ -247,11 +256,12 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
         }
 
         // O^T += V^T P^T ; V^T fragments come out of row-major V through transposing LDS reads
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const char* vp = sv + (ks * 16 + v_key) * ROWB + (((db * 4 + v_chunk) ^ v_sw) * 16) + v_in;
+                const char* vp = sk + ks * 16 * ROWB + v_addr[db];
                 const s16x4 lo = lds_read_tr(vp);
                 const s16x4 hi = lds_read_tr(vp + 8 * ROWB);
                 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -263,6 +273,7 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_kernel(AttnPa
             }
         }
 
+        __builtin_amdgcn_s_setprio(0);
         wait_all_vmem();   // this wave's part of the next tile has landed
         __syncthreads();   // everybody's has; and everybody is done reading this tile
     }
