@@ -37,6 +37,7 @@ struct GemmParams {
     int split_n, y2_col0, rows_per_batch;
     int act, act_begin;
     int tiles_m, tiles_n, group_m;
+    int bias_vec;  // 1: bias may be read with 8-byte buffer loads (4-byte aligned base)
     int vec_io;  // 1: every output/residual row segment of 8 columns may be accessed as 16 bytes
 };
 
@@ -48,10 +49,17 @@ constexpr uint32_t kOutOfRange = 0x80000000u;
 
 // LDS-direct buffer loads are counted by vmcnt; the workgroup barrier alone does not wait for them.
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// Two floats -> one dword of two bf16 (a in the low half): a single v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 __device__ __forceinline__ u32x2 pack4_bf16(float a, float b, float c, float d) {
     u32x2 r;
-    r.x = static_cast<uint32_t>(f2bf(a)) | (static_cast<uint32_t>(f2bf(b)) << 16);
-    r.y = static_cast<uint32_t>(f2bf(c)) | (static_cast<uint32_t>(f2bf(d)) << 16);
+    r.x = pack2_bf16(a, b);
+    r.y = pack2_bf16(c, d);
     return r;
 }
 
@@ -94,6 +102,256 @@ constexpr int load_at_slot(int g, int slots, int lps) {
     for (int l = 0; l < lps; ++l)
         if (l * slots / lps == g) return l;
     return -1;
+}
+
+// Epilogue shared by the tiled kernels. A lane's accumulators hold one activation row and runs of
+// 4 consecutive output columns. Per 32-row block: bias and GELU in fp32, one rounding to bf16, the
+// block is parked in LDS (a private region per wave, overlaying the ring, which the caller's final
+// barrier has retired) and leaves as 16-byte row segments, where the optional gated residual is
+// applied. Interior tiles with 16-byte addressable outputs take a branch-free path; edge tiles and
+// unaligned outputs take the checked path.
+__device__ __forceinline__ float tanh_gelu_fast(float x) {
+    // x * sigmoid(2u), u = sqrt(2/pi) (x + 0.044715 x^3), with log2(e) folded into the constants
+    const float x2 = x * x;
+    const float t = __builtin_fmaf(x2, -0.10294324f, -2.3022082f);
+    const float e = __builtin_amdgcn_exp2f(x * t);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+template <int MI, int NJ>
+__device__ __forceinline__ void gemm_epilogue_checked(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+                                                   int wave, int lane) {
+    constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
+    constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;  // bytes per row, 16-byte chunks per row
+    constexpr int RPI = 64 / C_CH;                         // rows one wave-wide 16-byte access covers
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    char* cw = lds + wave * (WROWS * C_PITCH);
+    const int wave_n0 = n0 + wn * WCOLS;
+    const int wave_m0 = m0 + wm * WROWS;
+
+    // bias for the lane's 4*NJ column quads
+    float bv[NJ][4][4];
+    const bool bias_fast = p.bias != nullptr && p.bias_vec;
+    if (bias_fast) {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + j * 32 + g * 8 + fhalf * 4) * 2, 0, 0);
+                bv[j][g][0] = __uint_as_float(raw.x << 16);
+                bv[j][g][1] = __uint_as_float(raw.x & 0xffff0000u);
+                bv[j][g][2] = __uint_as_float(raw.y << 16);
+                bv[j][g][3] = __uint_as_float(raw.y & 0xffff0000u);
+            }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int n = wave_n0 + j * 32 + g * 8 + fhalf * 4 + e;
+                    bv[j][g][e] = (p.bias != nullptr && n < p.N) ? bf2f(p.bias[n]) : 0.0f;
+                }
+    }
+
+    // LDS write address of column quad (j, g) in this lane's row, without the 32-row block offset
+    int waddr[NJ * 4];
+#pragma unroll
+    for (int c = 0; c < NJ * 4; ++c) waddr[c] = frow * C_PITCH + ((c ^ (frow & (C_CH - 1))) * 16) + fhalf * 8;
+    // read side: lane -> (row within the pass = lane / C_CH, chunk = lane % C_CH)
+    const int rrow = lane / C_CH, rch = lane % C_CH;
+
+    const bool gelu_all = p.act == FLUX_ACT_GELU_TANH && wave_n0 >= p.act_begin;
+    const bool gelu_some = p.act == FLUX_ACT_GELU_TANH && !gelu_all && wave_n0 + WCOLS > p.act_begin;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        // ---- accumulators of block row i -> bf16 -> LDS
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e] + bv[j][g][e];
+                if (gelu_all) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = tanh_gelu_fast(v[e]);
+                } else if (gelu_some) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (wave_n0 + j * 32 + g * 8 + fhalf * 4 + e >= p.act_begin) v[e] = tanh_gelu_fast(v[e]);
+                }
+                *reinterpret_cast<u32x2*>(cw + i * 32 * C_PITCH + waddr[j * 4 + g]) = pack4_bf16(v[0], v[1], v[2], v[3]);
+            }
+        __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
+
+        // ---- the 32 rows leave as 16-byte segments
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = i * 32 + it * RPI + rrow;
+            const int m = wave_m0 + row, n = wave_n0 + rch * 8;
+            Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + row * C_PITCH + ((rch ^ (row & (C_CH - 1))) * 16));
+            if (m >= p.M || n >= p.N) continue;
+            const bool full = p.vec_io && n + 8 <= p.N;
+            if (p.gate != nullptr) {
+                const bf16_t* gp = p.gate + static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n;
+                const bf16_t* rp = p.resid + static_cast<int64_t>(m) * p.ldresid + n;
+                if (full) {
+                    Vec16<bf16_t> gt = ld16(gp), rs = ld16(rp);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) y.v[e] = f2bf(bf2f(rs.v[e]) + bf2f(f2bf(bf2f(gt.v[e]) * bf2f(y.v[e]))));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (n + e < p.N) y.v[e] = f2bf(bf2f(rp[e]) + bf2f(f2bf(bf2f(gp[e]) * bf2f(y.v[e]))));
+                }
+            }
+            if (full && (n + 8 <= p.split_n || n >= p.split_n)) {
+                bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
+                                            : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
+                st16(dst, y);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int ne = n + e;
+                    if (ne < p.N) {
+                        bf16_t* dst = ne < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + ne
+                                                     : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (ne - p.split_n + p.y2_col0);
+                        *dst = y.v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Branch-free epilogue for interior tiles whose outputs (and residual operands) are 16-byte
+// addressable and whose columns all go to one destination. GELU is all-or-nothing for the wave.
+// Everything lane-dependent is computed once; per store only a wave-uniform row offset changes, so
+// the stores use a scalar base plus a 32-bit lane offset.
+template <int MI, int NJ, bool GELU, bool GATE>
+__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+                                                   int wave, int lane) {
+    constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
+    constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;
+    constexpr int RPI = 64 / C_CH;      // rows per wave-wide 16-byte access
+    constexpr int NIT = 32 / RPI;       // accesses per 32-row block
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    char* cw = lds + wave * (WROWS * C_PITCH);
+    const int wave_n0 = n0 + wn * WCOLS;
+    const int wave_m0 = m0 + wm * WROWS;
+
+    float bv[NJ][4][4];
+    if (p.bias != nullptr) {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + j * 32 + g * 8 + fhalf * 4) * 2, 0, 0);
+                bv[j][g][0] = __uint_as_float(raw.x << 16);
+                bv[j][g][1] = __uint_as_float(raw.x & 0xffff0000u);
+                bv[j][g][2] = __uint_as_float(raw.y << 16);
+                bv[j][g][3] = __uint_as_float(raw.y & 0xffff0000u);
+            }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) bv[j][g][e] = 0.0f;
+    }
+
+    int waddr[NJ * 4];
+#pragma unroll
+    for (int c = 0; c < NJ * 4; ++c) waddr[c] = frow * C_PITCH + ((c ^ (frow & (C_CH - 1))) * 16) + fhalf * 8;
+    const int rrow = lane / C_CH, rch = lane % C_CH;
+    // read address for access `it` of a block: row = it*RPI + rrow; the swizzle term repeats every 16 rows
+    constexpr int NSW = (16 / RPI) < NIT ? (16 / RPI) : NIT;
+    int raddr[NSW];
+#pragma unroll
+    for (int t = 0; t < NSW; ++t) {
+        const int row = t * RPI + rrow;
+        raddr[t] = row * C_PITCH + ((rch ^ (row & (C_CH - 1))) * 16);
+    }
+
+    const bool to_y = wave_n0 < p.split_n;
+    char* dst_u = reinterpret_cast<char*>(to_y ? p.Y + wave_n0 : p.Y2 + (wave_n0 - p.split_n + p.y2_col0));
+    const int64_t dst_ld = (to_y ? p.ldy : p.ldy2) * 2;            // bytes
+    const uint32_t dst_lane = static_cast<uint32_t>(rrow * dst_ld + rch * 16);
+    const char* res_u = nullptr;
+    const char* gate_u = nullptr;
+    uint32_t res_lane = 0;
+    if (GATE) {
+        res_u = reinterpret_cast<const char*>(p.resid + wave_n0);
+        res_lane = static_cast<uint32_t>(rrow * p.ldresid * 2 + rch * 16);
+        gate_u = reinterpret_cast<const char*>(p.gate + wave_n0 + rch * 8);
+    }
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = acc[i][j][g * 4 + e] + bv[j][g][e];
+                    if (GELU) v[e] = tanh_gelu_fast(v[e]);
+                }
+                *reinterpret_cast<u32x2*>(cw + i * 32 * C_PITCH + waddr[j * 4 + g]) = pack4_bf16(v[0], v[1], v[2], v[3]);
+            }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int row_u = i * 32 + it * RPI;                 // wave-uniform part of the row
+            Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + (i * 32 + (it / NSW) * NSW * RPI) * C_PITCH + raddr[it % NSW]);
+            const int64_t m_u = wave_m0 + row_u;
+            if (GATE) {
+                // all rows of one access belong to one batch element when rows_per_batch is a multiple of RPI
+                const Vec16<bf16_t> gt = ld16(reinterpret_cast<const bf16_t*>(gate_u) + ((m_u + rrow) / p.rows_per_batch) * p.gate_stride);
+                const Vec16<bf16_t> rs = *reinterpret_cast<const Vec16<bf16_t>*>(res_u + m_u * p.ldresid * 2 + res_lane);
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float y0 = bf2f(rs.v[e]) + bf2f(f2bf(bf2f(gt.v[e]) * bf2f(y.v[e])));
+                    const float y1 = bf2f(rs.v[e + 1]) + bf2f(f2bf(bf2f(gt.v[e + 1]) * bf2f(y.v[e + 1])));
+                    const uint32_t w = pack2_bf16(y0, y1);
+                    y.v[e] = static_cast<bf16_t>(w & 0xffffu);
+                    y.v[e + 1] = static_cast<bf16_t>(w >> 16);
+                }
+            }
+            *reinterpret_cast<Vec16<bf16_t>*>(dst_u + m_u * dst_ld + dst_lane) = y;
+        }
+    }
+}
+
+template <int MI, int NJ>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+                                              int wave, int lane) {
+    constexpr int BM = 64 * MI, BN = 64 * NJ, WCOLS = 32 * NJ;
+    const int wave_n0 = n0 + (wave & 1) * WCOLS;
+    const bool gelu_all = p.act == FLUX_ACT_GELU_TANH && wave_n0 >= p.act_begin;
+    const bool gelu_none = p.act != FLUX_ACT_GELU_TANH || wave_n0 + WCOLS <= p.act_begin;
+    const bool fast = p.vec_io && m0 + BM <= p.M && n0 + BN <= p.N && (gelu_all || gelu_none) &&
+                      (wave_n0 + WCOLS <= p.split_n || wave_n0 >= p.split_n) && (p.bias == nullptr || p.bias_vec) &&
+                      static_cast<int64_t>(BM) * p.ldy * 2 < 0x7fffffffLL && static_cast<int64_t>(BM) * p.ldy2 * 2 < 0x7fffffffLL;
+    if (fast) {
+        if (p.gate != nullptr) {
+            if (gelu_all) gemm_epilogue_fast<MI, NJ, true, true>(p, acc, lds, m0, n0, wave, lane);
+            else gemm_epilogue_fast<MI, NJ, false, true>(p, acc, lds, m0, n0, wave, lane);
+        } else {
+            if (gelu_all) gemm_epilogue_fast<MI, NJ, true, false>(p, acc, lds, m0, n0, wave, lane);
+            else gemm_epilogue_fast<MI, NJ, false, false>(p, acc, lds, m0, n0, wave, lane);
+        }
+    } else {
+        gemm_epilogue_checked<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+    }
 }
 
 template <int MI, int NJ, bool STAGED>
@@ -319,81 +577,171 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
         __syncthreads();
     }
 
-    // ---- epilogue phase 1: bias, rounding, GELU in accumulator layout -> bf16 tile in LDS (per wave)
-    char* cw = lds + wave * (WROWS * C_PITCH);
-    const int wave_n0 = n0 + wn * WCOLS;
-    const int wave_m0 = m0 + wm * WROWS;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int nl = j * 32 + g * 8 + fhalf * 4;  // first of 4 consecutive columns, wave-local
-            const int n = wave_n0 + nl;
-            float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (p.bias != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < p.N) bv[e] = bf2f(p.bias[n + e]);
-            }
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float t = acc[i][j][g * 4 + e] + bv[e];
-                    if (p.act == FLUX_ACT_GELU_TANH && n + e >= p.act_begin) t = gelu_tanh_f32(t);
-                    v[e] = t;
-                }
-                const int row = i * 32 + frow;
-                const int slot = (nl >> 3) ^ (row & (C_CH - 1));
-                *reinterpret_cast<u32x2*>(cw + row * C_PITCH + slot * 16 + fhalf * 8) = pack4_bf16(v[0], v[1], v[2], v[3]);
-            }
-        }
-    }
-    // The tile region is private to the wave (LDS operations of one wave complete in order), but
-    // the ring it overlays was shared: the barrier that ended the K loop already ordered every
-    // wave's last fragment reads before these writes.
-    __builtin_amdgcn_wave_barrier();
+    gemm_epilogue<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+}
 
-    // ---- epilogue phase 2: row-major 16-byte segments, optional gated residual, store
-    constexpr int SEGS = WROWS * C_CH;
-#pragma unroll 4
-    for (int it = 0; it < SEGS / 64; ++it) {
-        const int idx = it * 64 + lane;
-        const int row = idx / C_CH, ch = idx % C_CH;
-        const int m = wave_m0 + row, n = wave_n0 + ch * 8;
-        if (m >= p.M || n >= p.N) continue;
-        Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + row * C_PITCH + ((ch ^ (row & (C_CH - 1))) * 16));
-        const bool full = p.vec_io && n + 8 <= p.N;
-        if (p.gate != nullptr) {
-            const bf16_t* gp = p.gate + static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n;
-            const bf16_t* rp = p.resid + static_cast<int64_t>(m) * p.ldresid + n;
-            if (full) {
-                Vec16<bf16_t> g = ld16(gp), r = ld16(rp);
+// ------------------------------------------------------------------------------------------------
+// Paired-slab variant. The memory path of a CU moves 256-byte granules: asking for the two 128-byte
+// halves of a granule one K=64 slab apart (as the kernel above does) fetches every granule twice and
+// halves the achievable load rate. Here a thread loads both halves of a granule back to back (the
+// same rows, k and k+64) into registers, and the halves enter the two LDS stages when those become
+// free: stage 0 always holds the even slab (k % 128 < 64), stage 1 the odd one. One loop iteration
+// consumes a K=128 super-slab in eight K=16 steps with two barriers:
+//
+//   steps 0 1 2 | B1 | 3 4 5 6 | B2 | 7
+//   reads stage:  0 0 0   (3 reads 0, prefetches 1)  1 1 1   (7 reads 1, prefetches stage 0 of q+1)
+//   H1[l] -> stage 1 : step 7 of the previous iteration (l = 0..LPS/4-1) and steps 0..2   (half 1 of q)
+//   H0[l] -> stage 0 : steps 3..6                                                          (half 0 of q+1)
+//   right after H1[l] is stored, the pair (H0[l], H1[l]) of the following super-slab is requested;
+//   H0[l] is not stored before 4 steps later, H1[l] not before 8.
+// ------------------------------------------------------------------------------------------------
+template <int MI, int NJ>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_paired_kernel(GemmParams p) {
+    constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64;
+    constexpr int ROWB = BK * 2;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int PA = BM / 32, PB = BN / 32;
+    constexpr int LPS = PA + PB;                 // 16-byte chunks per thread per K=64 slab
+    constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
+    static_assert(4 * WROWS * WCOLS * 2 <= 2 * STAGE, "epilogue tile must fit the ring");
+    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+
+    int tm, tn;
+    if (!tile_of_block(p, tm, tn)) return;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // loader mapping (as in the kernel above): LDS slot (row = pass*32 + tid/8, position tid%8) holds
+    // logical chunk position ^ ((row>>1)&7)
+    const int lrow = tid >> 3;
+    const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
+    const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BN);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda), 0,
+        static_cast<int>(((rows_a - 1) * p.lda + p.K) * 2), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw), 0,
+        static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2), kRsrcFlags);
+    uint32_t voff[LPS];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) y.v[e] = f2bf(bf2f(r.v[e]) + bf2f(f2bf(bf2f(g.v[e]) * bf2f(y.v[e]))));
-            } else {
+    for (int i = 0; i < LPS; ++i) {
+        const int r = (i < PA ? i : i - PA) * 32 + lrow;
+        const bool ok = i < PA ? r < rows_a : r < rows_b;
+        const int64_t ld = i < PA ? p.lda : p.ldw;
+        voff[i] = ok ? static_cast<uint32_t>((r * ld + lchunk * 8) * 2) : kOutOfRange;
+    }
+    const int lds_slot = lrow * 128 + (tid & 7) * 16;
+
+    const int nq = (p.K + 2 * BK - 1) / (2 * BK);  // K=128 super-slabs
+    u32x4 h0[LPS], h1[LPS];
+    // Request chunk l of both halves of super-slab q. Chunks at or past K (K is a multiple of 8) and
+    // super-slabs past the end read as zeros.
+    auto load_pair = [&](int q, int l) {
+        const int k0 = q * (2 * BK) + lchunk * 8;
+        const uint32_t m0k = k0 >= p.K ? kOutOfRange : 0u;
+        const uint32_t m1k = k0 + BK >= p.K ? kOutOfRange : 0u;
+        const __amdgpu_buffer_rsrc_t rs = l < PA ? rsrc_a : rsrc_b;
+        h0[l] = load_chunk_reg(rs, voff[l] | m0k, q * (4 * BK));
+        h1[l] = load_chunk_reg(rs, voff[l] | m1k, q * (4 * BK) + 2 * BK);
+    };
+    auto store_half = [&](int stage, const u32x4& v, int l) {
+        char* dst = lds + stage * STAGE + lds_slot + (l < PA ? l * 4096 : A_BYTES + (l - PA) * 4096);
+        *reinterpret_cast<u32x4*>(dst) = v;
+    };
+
+    // fragment addressing
+    const int frow = lane & 31, fhalf = lane >> 5;
+    int koff[4];
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (n + e < p.N) y.v[e] = f2bf(bf2f(rp[e]) + bf2f(f2bf(bf2f(gp[e]) * bf2f(y.v[e]))));
-            }
-        }
-        if (full) {
-            bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
-                                        : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
-            st16(dst, y);
-        } else {
+    for (int kk = 0; kk < 4; ++kk) koff[kk] = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
+    const int a_off = (wm * WROWS + frow) * ROWB;
+    const int b_off = A_BYTES + (wn * WCOLS + frow) * ROWB;
+
+    f32x16 acc[MI][NJ];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int ne = n + e;
-                if (ne < p.N) {
-                    bf16_t* dst = ne < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + ne
-                                                 : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (ne - p.split_n + p.y2_col0);
-                    *dst = y.v[e];
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    bf16x8 xa[2][MI], wb[2][NJ];
+    auto read_frag = [&](int buf, const char* s, int kk, int r) {
+        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(s + a_off + koff[kk]);
+        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(s + b_off + (r - 1) * 32 * ROWB + koff[kk]);
+        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(s + a_off + (r - NJ) * 32 * ROWB + koff[kk]);
+    };
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / NJ, j = idx % NJ;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
+    };
+    constexpr int READS = MI + NJ, PER = (MI * NJ) / READS;
+    static_assert((MI * NJ) % READS == 0 && LPS % 4 == 0, "schedule shape");
+    constexpr int WPS = LPS / 4;  // register->LDS stores per step inside a 4-step window
+    // Step `stp` (0..7) of the iteration consuming super-slab q. Fragment reads of the next step are
+    // interleaved with this step's MFMAs; the store / load-pair actions sit in the first WPS slots.
+    auto step = [&](auto stp_c, int q) {
+        constexpr int STP = decltype(stp_c)::value;
+        constexpr int cur_buf = STP & 1;
+        constexpr int nstp = (STP + 1) & 7;
+        const char* nxt = lds + (nstp >> 2) * STAGE;
+#pragma unroll
+        for (int r = 0; r < READS; ++r) {
+            read_frag(cur_buf ^ 1, nxt, nstp & 3, r);
+            if (r < WPS) {
+                if constexpr (STP == 7) {            // half 1 of q+1, first quarter; then pairs of q+2
+                    store_half(1, h1[r], r);
+                    load_pair(q + 2, r);
+                } else if constexpr (STP <= 2) {     // half 1 of q, remaining quarters; then pairs of q+1
+                    const int l = (STP + 1) * WPS + r;
+                    store_half(1, h1[l], l);
+                    load_pair(q + 1, l);
+                } else {                             // steps 3..6: half 0 of q+1
+                    const int l = (STP - 3) * WPS + r;
+                    store_half(0, h0[l], l);
                 }
             }
+#pragma unroll
+            for (int m = 0; m < PER; ++m) mfma_one(cur_buf, r * PER + m);
+            __builtin_amdgcn_sched_barrier(0);
         }
+    };
+
+    // Prologue: super-slab 0 through the registers; its half 0 and the first quarter of its half 1 go
+    // to LDS, the freed registers take the pairs of super-slab 1.
+#pragma unroll
+    for (int l = 0; l < LPS; ++l) load_pair(0, l);
+#pragma unroll
+    for (int l = 0; l < LPS; ++l) store_half(0, h0[l], l);
+#pragma unroll
+    for (int l = 0; l < WPS; ++l) {
+        store_half(1, h1[l], l);
+        load_pair(1, l);
     }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
+    __builtin_amdgcn_sched_barrier(0);
+
+    for (int q = 0; q < nq; ++q) {
+        step(std::integral_constant<int, 0>{}, q);
+        step(std::integral_constant<int, 1>{}, q);
+        step(std::integral_constant<int, 2>{}, q);
+        __syncthreads();  // B1: half 1 of q is in stage 1
+        __builtin_amdgcn_sched_barrier(0);
+        step(std::integral_constant<int, 3>{}, q);
+        step(std::integral_constant<int, 4>{}, q);
+        step(std::integral_constant<int, 5>{}, q);
+        step(std::integral_constant<int, 6>{}, q);
+        __syncthreads();  // B2: half 0 of q+1 is in stage 0; stage 1 is free
+        __builtin_amdgcn_sched_barrier(0);
+        step(std::integral_constant<int, 7>{}, q);
+    }
+    __syncthreads();
+    gemm_epilogue<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -480,6 +828,17 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ, STAGED>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
+template <int MI, int NJ>
+static void launch_paired(GemmParams& p, hipStream_t st) {
+    constexpr int BM = 64 * MI, BN = 64 * NJ;
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    p.group_m = 4;
+    const int total = p.tiles_m * p.tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    hipLaunchKernelGGL((gemm_nt_paired_kernel<MI, NJ>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+}
+
 // Selected by FLUX_GEMM_VARIANT for experiments: 0 = automatic.
 static int gemm_variant() {
     static int v = [] {
@@ -518,6 +877,7 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     p.rows_per_batch = a->gate ? (int)a->rows_per_batch : 1;
     p.act = a->act; p.act_begin = (int)(a->act_begin < 0 ? 0 : (a->act_begin > a->N ? a->N : a->act_begin));
     p.tiles_m = p.tiles_n = 0; p.group_m = 4;
+    p.bias_vec = a->bias != nullptr && (reinterpret_cast<uintptr_t>(a->bias) & 3u) == 0 && a->N % 4 == 0;
     p.vec_io = aligned16(a->Y) && a->ldy % 8 == 0 &&
                (!split || (aligned16(a->Y2) && a->ldy2 % 8 == 0 && a->split_n % 8 == 0 && a->y2_col0 % 8 == 0)) &&
                (!a->gate || (aligned16(a->gate) && aligned16(a->resid) && a->ldresid % 8 == 0 && a->gate_batch_stride % 8 == 0));
@@ -545,6 +905,8 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     else if (variant == 2) launch_tiled<2, 2, false>(p, st);
     else if (variant == 3) launch_tiled<4, 4, true>(p, st);
     else if (variant == 4) launch_tiled<2, 2, true>(p, st);
+    else if (variant == 5) launch_paired<4, 4>(p, st);
+    else if (variant == 6) launch_paired<2, 2>(p, st);
     else if (big_tiles >= 192) launch_tiled<4, 4, false>(p, st);
     else launch_tiled<2, 2, false>(p, st);
     return check_launch("flux_linear_bf16");
