@@ -1,11 +1,10 @@
 // Linear layer on the matrix cores:  Y = epilogue(A[M,K] * W[N,K]^T), bf16 operands, fp32 accumulate.
 //
 // Both operands are K-contiguous, which is exactly what v_mfma_f32_32x32x16_bf16 wants: every lane
-// feeds 8 consecutive k of one row. A workgroup of four waves (2 x 2) owns a (64*MI) x (64*NJ) tile
-// of Y and each wave a (32*MI) x (32*NJ) sub-tile kept as MI*NJ accumulators of 32x32. The K loop
-// moves 64-wide slabs of A and W through a two-stage LDS ring: while the MFMAs consume stage s, the
-// slab for the next step lands in stage s^1 straight from buffer loads that write LDS (no register
-// staging).
+// feeds 8 consecutive k of one row. A workgroup of four waves (2 x 2) owns a (64*MI) x (64*MI) tile
+// of Y and each wave a (32*MI) x (32*MI) sub-tile kept as MI*MI accumulators of 32x32. The K loop
+// moves 64-wide slabs of A and W through a five-unit LDS ring (see the kernel) straight from buffer
+// loads that write LDS (no register staging).
 //
 // LDS slab layout: row r of the slab is 128 bytes = eight 16-byte chunks; chunk c is stored at
 // position c ^ ((r >> 1) & 7). LDS on gfx950 has 64 banks of 4 bytes, so a ds_read_b128 is served 16
@@ -15,8 +14,8 @@
 //
 // The MFMA takes W as its "A" operand and the activations as its "B" operand, so the accumulator
 // of a lane holds one activation row m and runs of 4 consecutive output columns n: bias and GELU
-// are applied there in fp32 and the result is rounded once, the bf16 tile goes through LDS once more and leaves as full 16-byte
-// row segments, where the optional gated residual is applied.
+// are applied there in fp32 and the result is rounded once; the bf16 tile goes through LDS once
+// more and leaves as full 16-byte row segments, where the optional gated residual is applied.
 #include "common.h"
 #include <stdlib.h>
 #include <type_traits>
@@ -89,20 +88,7 @@ __device__ __forceinline__ void load_chunk(__amdgpu_buffer_rsrc_t rsrc, char* ds
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soff, 0, 0);
 }
 
-__device__ __forceinline__ u32x4 load_chunk_reg(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, int soff) {
-    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
-}
-
 __device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-// Which of a slab's LPS buffer loads goes into issue slot g of SLOTS (-1 = none): spread evenly, so
-// the texture-address unit (64 bytes per clock per CU) is never asked for more than it can take and
-// the in-order wave does not stall MFMA issue behind a full memory queue.
-constexpr int load_at_slot(int g, int slots, int lps) {
-    for (int l = 0; l < lps; ++l)
-        if (l * slots / lps == g) return l;
-    return -1;
-}
 
 // Epilogue shared by the tiled kernels. A lane's accumulators hold one activation row and runs of
 // 4 consecutive output columns. Per 32-row block: bias and GELU in fp32, one rounding to bf16, the
@@ -354,257 +340,49 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     }
 }
 
-template <int MI, int NJ, bool STAGED>
-__global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(GemmParams p) {
-    constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64, NS = 2;
-    constexpr int ROWB = BK * 2;                 // bytes per slab row
-    constexpr int KSUB = BK / 16;                // MFMA K-steps per slab (4)
-    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
-    constexpr int PA = BM / 32, PB = BN / 32;    // loader passes per slab (32 rows = 4096 bytes each)
-    constexpr int LPS = PA + PB;                 // buffer loads per thread per slab
-    constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
-    constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;  // epilogue tile: bytes per row, 16-byte chunks per row
-    static_assert(4 * WROWS * C_PITCH <= NS * STAGE, "epilogue tile must fit the ring");
-    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
+// ------------------------------------------------------------------------------------------------
+// Tiled kernel: 64*MI x 64*MI output tile per workgroup of four waves (2 x 2, a wave owns
+// 32*MI x 32*MI), K in slabs of 64. With two whole-slab LDS stages the memory pipeline would drain
+// at every barrier (the wait in front of it is for ALL outstanding loads) and a slab's last loads
+// would get less than a K=16 step to land. Here LDS is a ring of five units, a unit holding one operand's share of a slab (BM rows x
+// 128 bytes): A(kt) lives in unit 2kt % 5 and W(kt) in unit (2kt+1) % 5. While slab kt is computed,
+// slab kt+1 and A(kt+2) occupy the other three units, so between two barriers the loads of W(kt+1)
+// and A(kt+2) are issued at an even pace, one per four MFMAs, and the wait in front of a barrier
+// only covers W(kt+1): the loads of A(kt+2) stay in flight across it. Every load has between half a
+// slab and a whole slab of MFMA time to land and the memory pipeline never runs empty.
+//
+//   slab kt :  step 0   step 1   step 2   step 3 = [MFMA x PER*BS] wait+barrier [rest, reads k0 of kt+1]
+//   loads   :  ......... G(kt) = W(kt+1), A(kt+2) ..........                    | G(kt+1) ...
+//
+// Ring offsets are wave-uniform scalars that advance by two units per slab.
+// ------------------------------------------------------------------------------------------------
+template <int K>
+using ic = std::integral_constant<int, K>;
 
-    int tm, tn;
-    if (!tile_of_block(p, tm, tn)) return;
-    const int m0 = tm * BM, n0 = tn * BN;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases in SGPRs
-    const int wm = wave >> 1, wn = wave & 1;
-
-    // ---- loader mapping: a wave's buffer load drops 64 x 16 bytes into 1 KB of consecutive LDS,
-    //      i.e. thread -> LDS slot (row = pass*32 + tid/8, position tid%8), so the thread fetches
-    //      logical chunk position ^ ((row>>1)&7) of that row from memory.
-    const int lrow = tid >> 3;
-    const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
-    const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BN);
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda), 0,
-        static_cast<int>(((rows_a - 1) * p.lda + p.K) * 2), kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw), 0,
-        static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2), kRsrcFlags);
-    uint32_t voff_a[PA], voff_b[PB];
-#pragma unroll
-    for (int i = 0; i < PA; ++i) {
-        const int r = i * 32 + lrow;
-        voff_a[i] = r < rows_a ? static_cast<uint32_t>((r * p.lda + lchunk * 8) * 2) : kOutOfRange;
-    }
-#pragma unroll
-    for (int i = 0; i < PB; ++i) {
-        const int r = i * 32 + lrow;
-        voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
-    }
-
-    const int nk = (p.K + BK - 1) / BK;
-    const bool k_ragged = (p.K % BK) != 0;
-    // The part of a slab past K is padded with zeros (K is a multiple of 8, so a 16-byte chunk is all
-    // in or all out).
-    auto slab_kmask = [&](int kt) -> uint32_t {
-        return (k_ragged && kt * BK + lchunk * 8 >= p.K) ? kOutOfRange : 0u;
-    };
-    // Register-staged path: slab data waits in registers (one 16-byte chunk per load) until its ring
-    // stage is free, which takes the memory pipeline off the critical path: a load issued in slot g
-    // is not needed before slot g of the next slab.
-    u32x4 sreg[STAGED ? LPS : 1];
-    const int lds_slot = lrow * 128 + (tid & 7) * 16;  // within a 32-row pass
-    auto stage_load = [&](int kt, int idx) {   // global -> sreg[idx]; slabs past the end read as zeros
-        const uint32_t kmask = (kt >= nk || (k_ragged && kt * BK + lchunk * 8 >= p.K)) ? kOutOfRange : 0u;
-        if (idx < PA) sreg[idx] = load_chunk_reg(rsrc_a, voff_a[idx] | kmask, kt * (BK * 2));
-        else sreg[idx] = load_chunk_reg(rsrc_b, voff_b[idx - PA] | kmask, kt * (BK * 2));
-    };
-    auto stage_store = [&](int kt, int idx) {  // sreg[idx] -> ring stage of slab kt
-        char* sa = lds + (kt & 1) * STAGE + lds_slot;
-        if (idx < PA) *reinterpret_cast<u32x4*>(sa + idx * 4096) = sreg[idx];
-        else *reinterpret_cast<u32x4*>(sa + A_BYTES + (idx - PA) * 4096) = sreg[idx];
-    };
-    // idx-th of the LPS buffer loads of slab kt: first the PA passes of A, then the PB passes of W
-    auto issue_load = [&](int kt, uint32_t kmask, int idx) {
-        char* sa = lds + (kt & 1) * STAGE + wave * 1024;
-        if (idx < PA) load_chunk(rsrc_a, sa + idx * 4096, voff_a[idx] | kmask, kt * (BK * 2));
-        else load_chunk(rsrc_b, sa + A_BYTES + (idx - PA) * 4096, voff_b[idx - PA] | kmask, kt * (BK * 2));
-    };
-
-    // ---- fragment addressing
-    const int frow = lane & 31, fhalf = lane >> 5;
-    int koff[KSUB];
-#pragma unroll
-    for (int kk = 0; kk < KSUB; ++kk) koff[kk] = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
-    const int a_off = (wm * WROWS + frow) * ROWB;
-    const int b_off = A_BYTES + (wn * WCOLS + frow) * ROWB;
-
-    f32x16 acc[MI][NJ];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    bf16x8 xa[2][MI], wb[2][NJ];  // two fragment sets: one feeds the MFMAs while the other is being read
-    auto read_frag = [&](int buf, const char* s, int kk, int r) {
-        // r-th fragment read of a step, in the order the MFMAs (activation block outer, weight
-        // block inner) first need them: x0, w0..w(NJ-1), x1..x(MI-1)
-        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(s + a_off + koff[kk]);
-        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(s + b_off + (r - 1) * 32 * ROWB + koff[kk]);
-        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(s + a_off + (r - NJ) * 32 * ROWB + koff[kk]);
-    };
-    auto mfma_one = [&](int buf, int idx) {
-        const int i = idx / NJ, j = idx % NJ;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
-    };
-    constexpr int READS = MI + NJ, MFMAS = MI * NJ, PER = MFMAS / READS;
-    static_assert(MFMAS % READS == 0, "MFMAs per fragment read");
-    // A slab's loads are issued over three K=16 steps: the step after the barrier that freed the
-    // stage (step 3 of the previous slab) and steps 0 and 1; step 2 stays free so that the loads have
-    // a few hundred cycles to land before the wait in front of the next barrier.
-    constexpr int SLOTS = 3 * READS;
-    // One K=16 step in a fixed interleave: every fragment read of the NEXT step is followed by PER
-    // MFMAs of the current one, so by the time a fragment is needed it was requested a whole step
-    // (>= 256 cycles) earlier; buffer loads of slab `load_kt` are dropped into their issue slots
-    // [slot0, slot0 + READS). The scheduling barriers pin this order; the compiler only adds the
-    // wait counts.
-    auto step = [&](int cur_buf, const char* nxt, int nxt_kk, auto has_next, auto slot0, int load_kt, uint32_t load_kmask) {
-#pragma unroll
-        for (int r = 0; r < READS; ++r) {
-            if constexpr (decltype(has_next)::value) read_frag(cur_buf ^ 1, nxt, nxt_kk, r);
-            constexpr int S0 = decltype(slot0)::value;
-            if constexpr (S0 >= 0 && !STAGED) {
-                const int l = load_at_slot(S0 + r, SLOTS, LPS);
-                if (l >= 0) issue_load(load_kt, load_kmask, l);
-            }
-            if constexpr (S0 >= 0 && STAGED) {
-                // load_kt = the slab whose chunk goes from registers to LDS in this slot; the freed
-                // register is refilled with the same chunk of the slab after it
-                const int l = load_at_slot(S0 + r, 4 * READS, LPS);
-                if (l >= 0) {
-                    stage_store(load_kt, l);
-                    stage_load(load_kt + 1, l);
-                }
-            }
-#pragma unroll
-            for (int m = 0; m < PER; ++m) mfma_one(cur_buf, r * PER + m);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    using no_loads = std::integral_constant<int, -1>;
-    // One slab with a successor. `more` says whether a slab kt+2 exists, whose first loads go out in
-    // the step after the barrier.
-    auto slab = [&](int kt, auto more) {
-        const char* s = lds + (kt & 1) * STAGE;
-        const char* sn = lds + ((kt & 1) ^ 1) * STAGE;
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (STAGED) {
-            // slots 8..31 move chunks of slab kt+1 into the other stage, the barrier publishes them
-            // and frees this slab's stage, whose first chunks (slab kt+2) follow in slots 0..7
-            step(0, s, 1, std::true_type{}, std::integral_constant<int, READS>{}, kt + 1, 0u);
-            step(1, s, 2, std::true_type{}, std::integral_constant<int, 2 * READS>{}, kt + 1, 0u);
-            step(0, s, 3, std::true_type{}, std::integral_constant<int, 3 * READS>{}, kt + 1, 0u);
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            step(1, sn, 0, std::true_type{}, std::integral_constant<int, 0>{}, kt + 2, 0u);
-            return;
-        }
-        const uint32_t kmask1 = slab_kmask(kt + 1);
-        step(0, s, 1, std::true_type{}, std::integral_constant<int, READS>{}, kt + 1, kmask1);
-        step(1, s, 2, std::true_type{}, std::integral_constant<int, 2 * READS>{}, kt + 1, kmask1);
-        step(0, s, 3, std::true_type{}, no_loads{}, 0, 0u);
-        wait_vmem_all();   // this wave's share of slab kt+1 has landed ...
-        __syncthreads();   // ... and so has everybody else's; all waves are done reading slab kt-1's stage
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (decltype(more)::value)
-            step(1, sn, 0, std::true_type{}, std::integral_constant<int, 0>{}, kt + 2, slab_kmask(kt + 2));
-        else
-            step(1, sn, 0, std::true_type{}, no_loads{}, 0, 0u);
-    };
-
-    if constexpr (STAGED) {
-        // Prologue: slab 0 through the registers into stage 0; slab 1 into the registers, and its
-        // chunks that belong to slots 0..7 already into stage 1.
-#pragma unroll
-        for (int i = 0; i < LPS; ++i) stage_load(0, i);
-#pragma unroll
-        for (int i = 0; i < LPS; ++i) stage_store(0, i);
-#pragma unroll
-        for (int i = 0; i < LPS; ++i) stage_load(1, i);
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
-#pragma unroll
-        for (int g = 0; g < READS; ++g) {
-            const int l = load_at_slot(g, 4 * READS, LPS);
-            if (l >= 0) {
-                stage_store(1, l);
-                stage_load(2, l);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    } else {
-    // Prologue: slab 0 completely, then the first third of slab 1.
-        const uint32_t km = slab_kmask(0);
-#pragma unroll
-        for (int i = 0; i < LPS; ++i) issue_load(0, km, i);
-        wait_vmem_all();
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
-        if (nk > 1) {
-            const uint32_t km1 = slab_kmask(1);
-#pragma unroll
-            for (int g = 0; g < READS; ++g) {
-                const int l = load_at_slot(g, SLOTS, LPS);
-                if (l >= 0) issue_load(1, km1, l);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-
-    int kt = 0;
-    for (; kt + 2 < nk; ++kt) slab(kt, std::true_type{});
-    if (kt + 1 < nk) {
-        slab(kt, std::false_type{});
-        ++kt;
-    }
-    {
-        const char* s = lds + (kt & 1) * STAGE;
-        step(0, s, 1, std::true_type{}, no_loads{}, 0, 0u);
-        step(1, s, 2, std::true_type{}, no_loads{}, 0, 0u);
-        step(0, s, 3, std::true_type{}, no_loads{}, 0, 0u);
-        step(1, nullptr, 0, std::false_type{}, no_loads{}, 0, 0u);
-        __syncthreads();
-    }
-
-    gemm_epilogue<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+template <int N>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+    // all but the newest N buffer loads of this wave have landed, its LDS reads have returned; the
+    // memory clobber keeps LDS accesses on their side of the barrier
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// ------------------------------------------------------------------------------------------------
-// Paired-slab variant. The memory path of a CU moves 256-byte granules: asking for the two 128-byte
-// halves of a granule one K=64 slab apart (as the kernel above does) fetches every granule twice and
-// halves the achievable load rate. Here a thread loads both halves of a granule back to back (the
-// same rows, k and k+64) into registers, and the halves enter the two LDS stages when those become
-// free: stage 0 always holds the even slab (k % 128 < 64), stage 1 the odd one. One loop iteration
-// consumes a K=128 super-slab in eight K=16 steps with two barriers:
-//
-//   steps 0 1 2 | B1 | 3 4 5 6 | B2 | 7
-//   reads stage:  0 0 0   (3 reads 0, prefetches 1)  1 1 1   (7 reads 1, prefetches stage 0 of q+1)
-//   H1[l] -> stage 1 : step 7 of the previous iteration (l = 0..LPS/4-1) and steps 0..2   (half 1 of q)
-//   H0[l] -> stage 0 : steps 3..6                                                          (half 0 of q+1)
-//   right after H1[l] is stored, the pair (H0[l], H1[l]) of the following super-slab is requested;
-//   H0[l] is not stored before 4 steps later, H1[l] not before 8.
-// ------------------------------------------------------------------------------------------------
-template <int MI, int NJ>
-__global__ __launch_bounds__(kGemmThreads) void gemm_nt_paired_kernel(GemmParams p) {
-    constexpr int BM = 64 * MI, BN = 64 * NJ, BK = 64;
-    constexpr int ROWB = BK * 2;
-    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
-    constexpr int PA = BM / 32, PB = BN / 32;
-    constexpr int LPS = PA + PB;                 // 16-byte chunks per thread per K=64 slab
+template <int MI>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p) {
+    constexpr int NJ = MI;
+    constexpr int BM = 64 * MI, BN = BM, BK = 64;
+    constexpr int ROWB = BK * 2, KSUB = BK / 16;
+    constexpr int UNIT = BM * ROWB, NU = 5;
+    constexpr int PU = BM / 32;                  // buffer loads per thread per unit
+    constexpr int NL = 2 * PU;                   // loads per group G(kt) = W(kt+1), A(kt+2)
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
-    static_assert(4 * WROWS * WCOLS * 2 <= 2 * STAGE, "epilogue tile must fit the ring");
-    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+    constexpr int READS = MI + NJ, MFMAS = MI * NJ, PER = MFMAS / READS;
+    constexpr int BS = READS / 4;                // slots of step 3 in front of the barrier
+    constexpr int NSLOT = KSUB * READS;          // issue slots per slab
+    constexpr int GB = 3 * READS + BS;           // first slot behind the barrier
+    constexpr int EARLY = NL - (GB + 1) / 2;     // loads of a group issued behind the previous slab's barrier
+    static_assert(MFMAS % READS == 0 && KSUB == 4 && NSLOT == 2 * NL, "schedule shape");
+    static_assert(4 * WROWS * WCOLS * 2 <= NU * UNIT, "epilogue tile must fit the ring");
+    __shared__ __attribute__((aligned(1024))) char lds[NU * UNIT];
 
     int tm, tn;
     if (!tile_of_block(p, tm, tn)) return;
@@ -614,8 +392,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_paired_kernel(GemmParams
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
-    // loader mapping (as in the kernel above): LDS slot (row = pass*32 + tid/8, position tid%8) holds
-    // logical chunk position ^ ((row>>1)&7)
+    // loader mapping: LDS slot (row = pass*32 + tid/8, position tid%8) holds logical chunk
+    // position ^ ((row>>1)&7) of that row
     const int lrow = tid >> 3;
     const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
     const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BN);
@@ -625,40 +403,42 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_paired_kernel(GemmParams
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw), 0,
         static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2), kRsrcFlags);
-    uint32_t voff[LPS];
+    uint32_t voff_a[PU], voff_b[PU];
 #pragma unroll
-    for (int i = 0; i < LPS; ++i) {
-        const int r = (i < PA ? i : i - PA) * 32 + lrow;
-        const bool ok = i < PA ? r < rows_a : r < rows_b;
-        const int64_t ld = i < PA ? p.lda : p.ldw;
-        voff[i] = ok ? static_cast<uint32_t>((r * ld + lchunk * 8) * 2) : kOutOfRange;
+    for (int i = 0; i < PU; ++i) {
+        const int r = i * 32 + lrow;
+        voff_a[i] = r < rows_a ? static_cast<uint32_t>((r * p.lda + lchunk * 8) * 2) : kOutOfRange;
+        voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
     }
-    const int lds_slot = lrow * 128 + (tid & 7) * 16;
-
-    const int nq = (p.K + 2 * BK - 1) / (2 * BK);  // K=128 super-slabs
-    u32x4 h0[LPS], h1[LPS];
-    // Request chunk l of both halves of super-slab q. Chunks at or past K (K is a multiple of 8) and
-    // super-slabs past the end read as zeros.
-    auto load_pair = [&](int q, int l) {
-        const int k0 = q * (2 * BK) + lchunk * 8;
-        const uint32_t m0k = k0 >= p.K ? kOutOfRange : 0u;
-        const uint32_t m1k = k0 + BK >= p.K ? kOutOfRange : 0u;
-        const __amdgpu_buffer_rsrc_t rs = l < PA ? rsrc_a : rsrc_b;
-        h0[l] = load_chunk_reg(rs, voff[l] | m0k, q * (4 * BK));
-        h1[l] = load_chunk_reg(rs, voff[l] | m1k, q * (4 * BK) + 2 * BK);
+    const int nk = (p.K + BK - 1) / BK;
+    const bool k_ragged = (p.K % BK) != 0;
+    // slabs past the end and the part of the last slab past K read as zeros
+    auto slab_mask = [&](int kt) -> uint32_t {
+        return (kt >= nk || (k_ragged && kt * BK + lchunk * 8 >= p.K)) ? kOutOfRange : 0u;
     };
-    auto store_half = [&](int stage, const u32x4& v, int l) {
-        char* dst = lds + stage * STAGE + lds_slot + (l < PA ? l * 4096 : A_BYTES + (l - PA) * 4096);
-        *reinterpret_cast<u32x4*>(dst) = v;
+    // ring offsets are wave-uniform byte offsets of a unit inside the ring
+    auto wrap = [&](int off) { return off >= NU * UNIT ? off - NU * UNIT : off; };
+    auto load_a = [&](int uoff, int pass, int kt, uint32_t mask) {
+        load_chunk(rsrc_a, lds + uoff + pass * 4096 + wave * 1024, voff_a[pass] | mask, kt * ROWB);
+    };
+    auto load_w = [&](int uoff, int pass, int kt, uint32_t mask) {
+        load_chunk(rsrc_b, lds + uoff + pass * 4096 + wave * 1024, voff_b[pass] | mask, kt * ROWB);
+    };
+    // load i of group G(kt) = W(kt+1) then A(kt+2); uw1 / ua2 are the units they go to
+    auto group_load = [&](int uw1, int ua2, int i, int kt, uint32_t m1, uint32_t m2) {
+        if (i < PU) load_w(uw1, i, kt + 1, m1);
+        else load_a(ua2, i - PU, kt + 2, m2);
     };
 
     // fragment addressing
     const int frow = lane & 31, fhalf = lane >> 5;
-    int koff[4];
+    int koff_a[KSUB], koff_w[KSUB];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) koff[kk] = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
-    const int a_off = (wm * WROWS + frow) * ROWB;
-    const int b_off = A_BYTES + (wn * WCOLS + frow) * ROWB;
+    for (int kk = 0; kk < KSUB; ++kk) {
+        const int ko = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
+        koff_a[kk] = (wm * WROWS + frow) * ROWB + ko;
+        koff_w[kk] = (wn * WCOLS + frow) * ROWB + ko;
+    }
 
     f32x16 acc[MI][NJ];
 #pragma unroll
@@ -669,77 +449,77 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_paired_kernel(GemmParams
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     bf16x8 xa[2][MI], wb[2][NJ];
-    auto read_frag = [&](int buf, const char* s, int kk, int r) {
-        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(s + a_off + koff[kk]);
-        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(s + b_off + (r - 1) * 32 * ROWB + koff[kk]);
-        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(s + a_off + (r - NJ) * 32 * ROWB + koff[kk]);
+    // r-th fragment of K-step kk of the slab whose units start at ua / uw, in the order the MFMAs
+    // first need them: x0, w0..w(NJ-1), x1..x(MI-1)
+    auto read_frag = [&](int buf, int ua, int uw, int kk, int r) {
+        const char* pa = lds + (ua + koff_a[kk]);
+        const char* pw = lds + (uw + koff_w[kk]);
+        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(pa);
+        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(pw + (r - 1) * 32 * ROWB);
+        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(pa + (r - NJ) * 32 * ROWB);
     };
     auto mfma_one = [&](int buf, int idx) {
         const int i = idx / NJ, j = idx % NJ;
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
     };
-    constexpr int READS = MI + NJ, PER = (MI * NJ) / READS;
-    static_assert((MI * NJ) % READS == 0 && LPS % 4 == 0, "schedule shape");
-    constexpr int WPS = LPS / 4;  // register->LDS stores per step inside a 4-step window
-    // Step `stp` (0..7) of the iteration consuming super-slab q. Fragment reads of the next step are
-    // interleaved with this step's MFMAs; the store / load-pair actions sit in the first WPS slots.
-    auto step = [&](auto stp_c, int q) {
-        constexpr int STP = decltype(stp_c)::value;
-        constexpr int cur_buf = STP & 1;
-        constexpr int nstp = (STP + 1) & 7;
-        const char* nxt = lds + (nstp >> 2) * STAGE;
+
+    // u = ring offset of A(kt)
+    auto slab = [&](int kt, int u) {
+        const int ua = u, uw = wrap(u + UNIT);                       // this slab
+        const int ua1 = wrap(u + 2 * UNIT), uw1 = wrap(u + 3 * UNIT);  // slab kt+1
+        const int ua2 = wrap(u + 4 * UNIT), uw2 = u;                   // slab kt+2 (W takes this slab's A unit)
+        const uint32_t m1 = slab_mask(kt + 1), m2 = slab_mask(kt + 2);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int r = 0; r < READS; ++r) {
-            read_frag(cur_buf ^ 1, nxt, nstp & 3, r);
-            if (r < WPS) {
-                if constexpr (STP == 7) {            // half 1 of q+1, first quarter; then pairs of q+2
-                    store_half(1, h1[r], r);
-                    load_pair(q + 2, r);
-                } else if constexpr (STP <= 2) {     // half 1 of q, remaining quarters; then pairs of q+1
-                    const int l = (STP + 1) * WPS + r;
-                    store_half(1, h1[l], l);
-                    load_pair(q + 1, l);
-                } else {                             // steps 3..6: half 0 of q+1
-                    const int l = (STP - 3) * WPS + r;
-                    store_half(0, h0[l], l);
-                }
+        for (int s = 0; s < NSLOT; ++s) {
+            const int stp = s / READS, r = s % READS;
+            if (s == GB) {
+                wait_loads_and_barrier<PU>();  // slab kt+1 is complete in LDS; this slab's units are free
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (stp < 3) {
+                read_frag((stp & 1) ^ 1, ua, uw, stp + 1, r);
+            } else if (r >= BS) {
+                const int rr = r - BS;
+                const int lo = rr + (rr < BS ? rr : BS), n = rr < BS ? 2 : 1;
+                for (int f = lo; f < lo + n; ++f) read_frag(0, ua1, uw1, 0, f);
+            }
+            if (s % 2 == 0) {
+                if (s < GB) group_load(uw1, ua2, EARLY + s / 2, kt, m1, m2);
+                else load_w(uw2, (s - GB - GB % 2) / 2, kt + 2, m2);  // first loads of G(kt+1)
             }
 #pragma unroll
-            for (int m = 0; m < PER; ++m) mfma_one(cur_buf, r * PER + m);
+            for (int m = 0; m < PER; ++m) mfma_one(stp & 1, r * PER + m);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // Prologue: super-slab 0 through the registers; its half 0 and the first quarter of its half 1 go
-    // to LDS, the freed registers take the pairs of super-slab 1.
+    // Prologue: slab 0, A(1) and the first loads of G(0); slab 0 must have landed, the rest flies on.
+    {
+        const uint32_t k0 = slab_mask(0), k1 = slab_mask(1);
 #pragma unroll
-    for (int l = 0; l < LPS; ++l) load_pair(0, l);
+        for (int i = 0; i < PU; ++i) load_a(0, i, 0, k0);
 #pragma unroll
-    for (int l = 0; l < LPS; ++l) store_half(0, h0[l], l);
+        for (int i = 0; i < PU; ++i) load_w(UNIT, i, 0, k0);
 #pragma unroll
-    for (int l = 0; l < WPS; ++l) {
-        store_half(1, h1[l], l);
-        load_pair(1, l);
+        for (int i = 0; i < PU; ++i) load_a(2 * UNIT, i, 1, k1);
+#pragma unroll
+        for (int i = 0; i < EARLY; ++i) load_w(3 * UNIT, i, 1, k1);
+        wait_loads_and_barrier<PU + EARLY>();
+#pragma unroll
+        for (int r = 0; r < READS; ++r) read_frag(0, 0, UNIT, 0, r);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < READS; ++r) read_frag(0, lds, 0, r);
-    __builtin_amdgcn_sched_barrier(0);
+    static_assert(EARLY <= PU, "loads behind the barrier must all belong to W");
 
-    for (int q = 0; q < nq; ++q) {
-        step(std::integral_constant<int, 0>{}, q);
-        step(std::integral_constant<int, 1>{}, q);
-        step(std::integral_constant<int, 2>{}, q);
-        __syncthreads();  // B1: half 1 of q is in stage 1
-        __builtin_amdgcn_sched_barrier(0);
-        step(std::integral_constant<int, 3>{}, q);
-        step(std::integral_constant<int, 4>{}, q);
-        step(std::integral_constant<int, 5>{}, q);
-        step(std::integral_constant<int, 6>{}, q);
-        __syncthreads();  // B2: half 0 of q+1 is in stage 0; stage 1 is free
-        __builtin_amdgcn_sched_barrier(0);
-        step(std::integral_constant<int, 7>{}, q);
+    int u = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        slab(kt, u);
+        u = wrap(u + 2 * UNIT);
     }
+    // The last slab's trailing loads were masked (they move no data but still write zeros to LDS):
+    // retire them before the epilogue reuses the ring.
+    wait_vmem_all();
     __syncthreads();
     gemm_epilogue<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
 }
@@ -817,32 +597,21 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     *dst = f2bf(t);
 }
 
-template <int MI, int NJ, bool STAGED>
+template <int MI>
 static void launch_tiled(GemmParams& p, hipStream_t st) {
-    constexpr int BM = 64 * MI, BN = 64 * NJ;
+    constexpr int BM = 64 * MI;
     p.tiles_m = (p.M + BM - 1) / BM;
-    p.tiles_n = (p.N + BN - 1) / BN;
+    p.tiles_n = (p.N + BM - 1) / BM;
     p.group_m = 4;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((gemm_nt_kernel<MI, NJ, STAGED>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    hipLaunchKernelGGL((gemm_nt_ring_kernel<MI>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
-template <int MI, int NJ>
-static void launch_paired(GemmParams& p, hipStream_t st) {
-    constexpr int BM = 64 * MI, BN = 64 * NJ;
-    p.tiles_m = (p.M + BM - 1) / BM;
-    p.tiles_n = (p.N + BN - 1) / BN;
-    p.group_m = 4;
-    const int total = p.tiles_m * p.tiles_n;
-    const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((gemm_nt_paired_kernel<MI, NJ>), dim3(grid), dim3(kGemmThreads), 0, st, p);
-}
-
-// Selected by FLUX_GEMM_VARIANT for experiments: 0 = automatic.
-static int gemm_variant() {
+// FLUX_GEMM_TILE=256 or 128 forces the tile size (for measurements); anything else = automatic.
+static int forced_tile() {
     static int v = [] {
-        const char* e = getenv("FLUX_GEMM_VARIANT");
+        const char* e = getenv("FLUX_GEMM_TILE");
         return e ? atoi(e) : 0;
     }();
     return v;
@@ -899,15 +668,11 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
         hipLaunchKernelGGL((gemv_small_m_kernel<8>), dim3((unsigned)((p.N + 3) / 4)), dim3(256), 0, st, p);
         return check_launch("flux_linear_bf16");
     }
-    const int variant = gemm_variant();
+    // 256 x 256 tiles once they fill most of the 256 CUs; below that 128 x 128 tiles (two workgroups
+    // per CU) spread the work better than they lose in operand re-reads.
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-    if (variant == 1) launch_tiled<4, 4, false>(p, st);
-    else if (variant == 2) launch_tiled<2, 2, false>(p, st);
-    else if (variant == 3) launch_tiled<4, 4, true>(p, st);
-    else if (variant == 4) launch_tiled<2, 2, true>(p, st);
-    else if (variant == 5) launch_paired<4, 4>(p, st);
-    else if (variant == 6) launch_paired<2, 2>(p, st);
-    else if (big_tiles >= 192) launch_tiled<4, 4, false>(p, st);
-    else launch_tiled<2, 2, false>(p, st);
+    const int tile = forced_tile();
+    if (tile == 256 || (tile != 128 && big_tiles >= 160)) launch_tiled<4>(p, st);
+    else launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
 }
