@@ -411,13 +411,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
         voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
     }
     const int nk = (p.K + BK - 1) / BK;
-    const bool k_ragged = (p.K % BK) != 0;
-    // slabs past the end and the part of the last slab past K read as zeros
-    auto slab_mask = [&](int kt) -> uint32_t {
-        return (kt >= nk || (k_ragged && kt * BK + lchunk * 8 >= p.K)) ? kOutOfRange : 0u;
-    };
+    // Slabs past the end and the part of the last slab past K read as zeros: both are "this
+    // thread's chunk starts at or past K" (K is a multiple of 8, so a chunk is all in or all out).
+    auto slab_mask = [&](int kt) -> uint32_t { return kt * BK + lchunk * 8 >= p.K ? kOutOfRange : 0u; };
     // ring offsets are wave-uniform byte offsets of a unit inside the ring
-    auto wrap = [&](int off) { return off >= NU * UNIT ? off - NU * UNIT : off; };
     auto load_a = [&](int uoff, int pass, int kt, uint32_t mask) {
         load_chunk(rsrc_a, lds + uoff + pass * 4096 + wave * 1024, voff_a[pass] | mask, kt * ROWB);
     };
@@ -463,12 +460,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
     };
 
-    // u = ring offset of A(kt)
-    auto slab = [&](int kt, int u) {
-        const int ua = u, uw = wrap(u + UNIT);                       // this slab
-        const int ua1 = wrap(u + 2 * UNIT), uw1 = wrap(u + 3 * UNIT);  // slab kt+1
-        const int ua2 = wrap(u + 4 * UNIT), uw2 = u;                   // slab kt+2 (W takes this slab's A unit)
-        const uint32_t m1 = slab_mask(kt + 1), m2 = slab_mask(kt + 2);
+    // ua/uw: units of slab kt, ua1/uw1: of slab kt+1, ua2: of A(kt+2); W(kt+2) takes over ua once
+    // the barrier has retired it. m1/m2: load masks of slabs kt+1 / kt+2; the mask of slab kt+3 is
+    // worked out in the shadow of an MFMA so that the loop back-edge carries register moves only.
+    auto slab = [&](int kt, int ua, int uw, int ua1, int uw1, int ua2, uint32_t m1, uint32_t m2, uint32_t& m3) {
+        const int uw2 = ua;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < NSLOT; ++s) {
@@ -484,12 +480,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
                 const int lo = rr + (rr < BS ? rr : BS), n = rr < BS ? 2 : 1;
                 for (int f = lo; f < lo + n; ++f) read_frag(0, ua1, uw1, 0, f);
             }
+            // one memory instruction per MFMA interval: the fragment read goes in front of the slot's
+            // first MFMA, the buffer load behind it
+            mfma_one(stp & 1, r * PER);
+            if (s == 1) m3 = slab_mask(kt + 3);
+            __builtin_amdgcn_sched_barrier(0);
             if (s % 2 == 0) {
                 if (s < GB) group_load(uw1, ua2, EARLY + s / 2, kt, m1, m2);
                 else load_w(uw2, (s - GB - GB % 2) / 2, kt + 2, m2);  // first loads of G(kt+1)
             }
 #pragma unroll
-            for (int m = 0; m < PER; ++m) mfma_one(stp & 1, r * PER + m);
+            for (int m = 1; m < PER; ++m) mfma_one(stp & 1, r * PER + m);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -512,10 +513,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     }
     static_assert(EARLY <= PU, "loads behind the barrier must all belong to W");
 
-    int u = 0;
-    for (int kt = 0; kt < nk; ++kt) {
-        slab(kt, u);
-        u = wrap(u + 2 * UNIT);
+    {
+        int ua = 0, uw = UNIT, ua1 = 2 * UNIT, uw1 = 3 * UNIT, ua2 = 4 * UNIT;
+        uint32_t m1 = slab_mask(1), m2 = slab_mask(2);
+        for (int kt = 0; kt < nk; ++kt) {
+            uint32_t m3;
+            slab(kt, ua, uw, ua1, uw1, ua2, m1, m2, m3);
+            // the ring advances by two units
+            const int t0 = ua, t1 = uw;
+            ua = ua1; uw = uw1; ua1 = ua2; uw1 = t0; ua2 = t1;
+            m1 = m2; m2 = m3;
+        }
     }
     // The last slab's trailing loads were masked (they move no data but still write zeros to LDS):
     // retire them before the epilogue reuses the ring.
