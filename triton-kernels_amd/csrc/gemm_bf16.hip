@@ -476,9 +476,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
             if (stp < 3) {
                 read_frag((stp & 1) ^ 1, ua, uw, stp + 1, r);
             } else if (r >= BS) {
-                const int rr = r - BS;
-                const int lo = rr + (rr < BS ? rr : BS), n = rr < BS ? 2 : 1;
-                for (int f = lo; f < lo + n; ++f) read_frag(0, ua1, uw1, 0, f);
+                // two per slot: the last one is requested a few MFMAs before the slab ends, so the
+                // wait at the top of the next slab finds it done
+                const int lo = 2 * (r - BS);
+                for (int f = lo; f < lo + 2 && f < READS; ++f) read_frag(0, ua1, uw1, 0, f);
             }
             // one memory instruction per MFMA interval: the fragment read goes in front of the slot's
             // first MFMA, the buffer load behind it
