@@ -5,8 +5,7 @@
 // A row of D elements is owned by D/VEC adjacent lanes (16 lanes for D = 128 in bf16), each holding
 // one 16-byte vector = VEC/2 rotation pairs, so the per-row reduction is a DPP butterfly and the
 // rotation needs no cross-lane traffic. q and k of the same (b,h,s) are handled by the same lane
-// and share the pe registers. Blocks walk the sequence fastest, so the tile of pe a block needs is
-// the same for every head and stays in the L2 of the XCD that keeps getting that tile.
+// and share the pe registers, and so do four consecutive heads.
 #include "common.h"
 
 namespace flux {
@@ -26,28 +25,51 @@ struct PrepParams {
     int64_t pe_sb;
     int64_t H, Lt, L;
     float eps;
+    int scale_vec;  // 1: every RMS scale pointer is 16-byte aligned (vector loads)
 };
 
+// Row of source s at (b, h, pos): txt rows first, then img rows. Both candidates are formed and one
+// is selected, so there is no branch in front of the load.
 template <typename T>
-__device__ __forceinline__ const T* src_row(const Src& s, int64_t b, int64_t h, int64_t pos, int64_t Lt, bool& is_txt) {
-    is_txt = pos < Lt;
-    if (is_txt) return static_cast<const T*>(s.txt) + b * s.t_sb + h * s.t_sh + pos * s.t_sl;
-    return static_cast<const T*>(s.img) + b * s.i_sb + h * s.i_sh + (pos - Lt) * s.i_sl;
+__device__ __forceinline__ const T* src_row(const Src& s, int64_t b, int64_t h, int64_t pos, int64_t Lt) {
+    const T* t = static_cast<const T*>(s.txt) + b * s.t_sb + h * s.t_sh + pos * s.t_sl;
+    const T* i = static_cast<const T*>(s.img) + b * s.i_sb + h * s.i_sh + (pos - Lt) * s.i_sl;
+    return pos < Lt ? t : i;
 }
 
+// Heads one thread walks with the same pe / scale registers: the rotation table is read once per
+// position and head group instead of once per head, which cuts its share of the L2 traffic from as
+// much as q and k together to a quarter of that.
+constexpr int kHeadGroup = 4;
+
+// The kernel is straight-line code: rows past the end of the sequence and heads past the last one
+// are clamped to the last valid row / head for the loads and only the stores are predicated, so
+// every load of a thread (pe, scales, the head group's q and k vectors) is in flight before the
+// first one is consumed.
 template <typename T, typename TS, int D, bool NORM, bool ROPE>
 __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int G = (D / VEC) < 64 ? (D / VEC) : 64;   // lanes per row
     constexpr int ITER = D / (VEC * G);                   // 16-byte vectors per lane
     constexpr int ROWS = kPrepBlock / G;
+    constexpr int HG = ITER == 1 ? kHeadGroup : 1;        // long rows already give a thread enough loads in flight
     static_assert(G * ITER * VEC == D, "head dim must be a multiple of the vector width");
     const int lane = threadIdx.x % G;
-    const int64_t pos = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / G;
-    const int64_t bh = blockIdx.y;
-    const int64_t b = bh / p.H, h = bh % p.H;
-    const bool ok = pos < p.L;
-    const int64_t out_row = (bh * p.L + pos) * D;
+    // the head group is the fastest-moving block coordinate: blocks in flight together read whole
+    // source rows (all heads of a position are adjacent in a fused qkv projection)
+    const int64_t groups = (p.H + HG - 1) / HG;
+    const int64_t pos_raw = static_cast<int64_t>(blockIdx.x / groups) * ROWS + threadIdx.x / G;
+    const int64_t b = blockIdx.y, h0 = (blockIdx.x % groups) * HG;
+    const bool ok = pos_raw < p.L;
+    const int64_t pos = ok ? pos_raw : p.L - 1;
+    const bool is_txt = pos < p.Lt;
+    int64_t hh[HG];
+    bool hok[HG];
+#pragma unroll
+    for (int g = 0; g < HG; ++g) {
+        hok[g] = ok && h0 + g < p.H;
+        hh[g] = h0 + g < p.H ? h0 + g : p.H - 1;
+    }
 
     // pe[pos, pair, a, j]: the lane's vector at column c covers pairs c/2 .. c/2 + VEC/2 - 1
     float f[ITER][VEC * 2];
@@ -55,95 +77,119 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
 #pragma unroll
         for (int it = 0; it < ITER; ++it) {
             const int c = (it * G + lane) * VEC;
-            if (ok) {
-                const float* fp = p.pe + b * p.pe_sb + pos * (2 * D) + c * 2;
+            const float* fp = p.pe + b * p.pe_sb + pos * (2 * D) + c * 2;
 #pragma unroll
-                for (int i = 0; i < VEC * 2 / 4; ++i) {
-                    Vec16<float> t = ld16(fp + i * 4);
+            for (int i = 0; i < VEC * 2 / 4; ++i) {
+                Vec16<float> t = ld16(fp + i * 4);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) f[it][i * 4 + e] = t.v[e];
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < VEC * 2; ++i) f[it][i] = 0.0f;
+                for (int e = 0; e < 4; ++e) f[it][i * 4 + e] = t.v[e];
             }
         }
     }
 
     // v: bit-exact copy
-    if (p.v.out != nullptr && ok) {
-        bool is_txt;
-        const T* src = src_row<T>(p.v, b, h, pos, p.Lt, is_txt);
+    if (p.v.out != nullptr) {
+        Vec16<T> vv[HG][ITER];
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) {
-            const int c = (it * G + lane) * VEC;
-            st16(static_cast<T*>(p.v.out) + out_row + c, ld16(src + c));
+        for (int g = 0; g < HG; ++g) {
+            const T* src = src_row<T>(p.v, b, hh[g], pos, p.Lt);
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) vv[g][it] = ld16(src + (it * G + lane) * VEC);
+        }
+#pragma unroll
+        for (int g = 0; g < HG; ++g) {
+            T* out = static_cast<T*>(p.v.out) + ((b * p.H + hh[g]) * p.L + pos) * D;
+            if (hok[g]) {
+#pragma unroll
+                for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, vv[g][it]);
+            }
+        }
+    }
+
+    // all q and k loads of the head group go out before the first one is used
+    Vec16<T> raw[2][HG][ITER];
+    float w[2][ITER][VEC];
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const Src& s = which == 0 ? p.q : p.k;
+        if (s.out == nullptr) continue;  // uniform over the grid
+#pragma unroll
+        for (int g = 0; g < HG; ++g) {
+            const T* src = src_row<T>(s, b, hh[g], pos, p.Lt);
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) raw[which][g][it] = ld16(src + (it * G + lane) * VEC);
+        }
+        if (NORM) {
+            const TS* sc = static_cast<const TS*>(is_txt ? s.scale_txt : s.scale_img);
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const TS* sp = sc + (it * G + lane) * VEC;
+                if (p.scale_vec) {
+#pragma unroll
+                    for (int i = 0; i < VEC / Elem<TS>::VEC; ++i) {
+                        const Vec16<TS> t = ld16(sp + i * Elem<TS>::VEC);
+#pragma unroll
+                        for (int e = 0; e < Elem<TS>::VEC; ++e) w[which][it][i * Elem<TS>::VEC + e] = Elem<TS>::load(t.v[e]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) w[which][it][e] = Elem<TS>::load(sp[e]);
+                }
+            }
         }
     }
 
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
         const Src& s = which == 0 ? p.q : p.k;
-        if (s.out == nullptr) continue;  // uniform over the grid
-        T* out = static_cast<T*>(s.out) + out_row;
-        bool is_txt = false;
-        Vec16<T> raw[ITER];
-        if (ok) {
-            const T* src = src_row<T>(s, b, h, pos, p.Lt, is_txt);
+        if (s.out == nullptr) continue;
 #pragma unroll
-            for (int it = 0; it < ITER; ++it) raw[it] = ld16(src + (it * G + lane) * VEC);
-        } else {
+        for (int g = 0; g < HG; ++g) {
+            T* out = static_cast<T*>(s.out) + ((b * p.H + hh[g]) * p.L + pos) * D;
+            if (!NORM && !ROPE) {
+                if (hok[g]) {
 #pragma unroll
-            for (int it = 0; it < ITER; ++it)
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) raw[it].v[e] = T(0);
-        }
-        if (!NORM && !ROPE) {
-            if (ok) {
-#pragma unroll
-                for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, raw[it]);
+                    for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, raw[which][g][it]);
+                }
+                continue;
             }
-            continue;
-        }
-        float x[ITER][VEC];
-#pragma unroll
-        for (int it = 0; it < ITER; ++it)
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) x[it][e] = Elem<T>::load(raw[it].v[e]);
-        if (NORM) {
-            float ss = 0.0f;
+            float x[ITER][VEC];
 #pragma unroll
             for (int it = 0; it < ITER; ++it)
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) ss += x[it][e] * x[it][e];
-            ss = group_sum<G>(ss);  // every lane of the wave takes part, rows past the end hold zeros
-            const float rstd = rsqrtf(ss / static_cast<float>(D) + p.eps);
-            const TS* sc = static_cast<const TS*>(is_txt ? s.scale_txt : s.scale_img);
+                for (int e = 0; e < VEC; ++e) x[it][e] = Elem<T>::load(raw[which][g][it].v[e]);
+            if (NORM) {
+                float ss = 0.0f;
+#pragma unroll
+                for (int it = 0; it < ITER; ++it)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) ss += x[it][e] * x[it][e];
+                ss = group_sum<G>(ss);
+                const float rstd = rsqrtf(ss / static_cast<float>(D) + p.eps);
+#pragma unroll
+                for (int it = 0; it < ITER; ++it)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) x[it][e] = Elem<T>::round(Elem<T>::round(x[it][e] * rstd) * w[which][it][e]);
+            }
+            Vec16<T> o[ITER];
 #pragma unroll
             for (int it = 0; it < ITER; ++it) {
-                const int c = (it * G + lane) * VEC;
+                if (ROPE) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float w = ok ? Elem<TS>::load(sc[c + e]) : 0.0f;
-                    x[it][e] = Elem<T>::round(Elem<T>::round(x[it][e] * rstd) * w);
+                    for (int i = 0; i < VEC / 2; ++i) {
+                        const float x0 = x[it][2 * i], x1 = x[it][2 * i + 1];
+                        o[it].v[2 * i] = Elem<T>::store(f[it][4 * i + 0] * x0 + f[it][4 * i + 1] * x1);
+                        o[it].v[2 * i + 1] = Elem<T>::store(f[it][4 * i + 2] * x0 + f[it][4 * i + 3] * x1);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) o[it].v[e] = Elem<T>::store(x[it][e]);
                 }
             }
-        }
+            if (hok[g]) {
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) {
-            Vec16<T> o;
-            if (ROPE) {
-#pragma unroll
-                for (int i = 0; i < VEC / 2; ++i) {
-                    const float x0 = x[it][2 * i], x1 = x[it][2 * i + 1];
-                    o.v[2 * i] = Elem<T>::store(f[it][4 * i + 0] * x0 + f[it][4 * i + 1] * x1);
-                    o.v[2 * i + 1] = Elem<T>::store(f[it][4 * i + 2] * x0 + f[it][4 * i + 3] * x1);
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) o.v[e] = Elem<T>::store(x[it][e]);
+                for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, o[it]);
             }
-            if (ok) st16(out + (it * G + lane) * VEC, o);
         }
     }
 }
@@ -189,12 +235,18 @@ static int prep_launch(const flux_qkv_prep_args& a, hipStream_t st) {
     p.pe = a.pe;
     p.pe_sb = a.pe_batch_stride;
     p.H = a.H; p.Lt = a.Lt; p.L = L; p.eps = a.eps;
+    p.scale_vec = 1;
+    for (int i = 0; i < 2; ++i)
+        if ((sc_t[i] && !aligned16(sc_t[i])) || (sc_i[i] && !aligned16(sc_i[i]))) p.scale_vec = 0;
 
     const int D = a.D;
     const int lanes_per_row = D / VEC < 64 ? D / VEC : 64;
     const int rows_per_block = kPrepBlock / (lanes_per_row > 0 ? lanes_per_row : 1);
-    dim3 grid((unsigned)((L + rows_per_block - 1) / rows_per_block), (unsigned)(a.B * a.H));
-    if (a.B * a.H > 65535) return fail(FLUX_E_SHAPE, "flux_qkv_prep: B*H = %lld exceeds 65535", (long long)(a.B * a.H));
+    // rows of one 16-byte vector per lane are walked kHeadGroup heads at a time (see the kernel)
+    const int64_t hg = (D / VEC <= 64) ? kHeadGroup : 1;
+    const int64_t pos_blocks = (L + rows_per_block - 1) / rows_per_block, groups = (a.H + hg - 1) / hg;
+    if (a.B > 65535 || pos_blocks * groups > 0x7fffffffLL) return fail(FLUX_E_SHAPE, "flux_qkv_prep: grid too large (B=%lld, L=%lld, H=%lld)", (long long)a.B, (long long)L, (long long)a.H);
+    dim3 grid((unsigned)(pos_blocks * groups), (unsigned)a.B);
 
 #define LAUNCH(D_, N_, R_) hipLaunchKernelGGL((qkv_prep_kernel<T, TS, D_, N_, R_>), grid, dim3(kPrepBlock), 0, st, p)
 #define BY_FLAGS(D_)                                   \
