@@ -535,50 +535,88 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
 
 // ------------------------------------------------------------------------------------------------
 // Skinny problems (M <= 8, e.g. the Modulation projection of one conditioning vector per batch
-// element): HBM-bound on W. One wave per output column streams the W row with 16-byte loads while
-// the few activation rows come from cache; the dot products are folded with a wave butterfly.
+// element): HBM-bound on W. A wave streams the W rows of two output columns with 16-byte loads,
+// six in flight per lane, while the few activation rows come from cache; the dot products are
+// folded with a wave butterfly. The kernel is instantiated per row count, so it has no row tests.
 // ------------------------------------------------------------------------------------------------
-template <int MMAX>
+constexpr int kGemvCols = 2;  // output columns per wave
+
+template <int MM>
 __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
+    constexpr int CPW = kGemvCols, U = 3;  // CPW * U 16-byte loads of W in flight per lane
     const int lane = threadIdx.x & 63;
-    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (n >= p.N) return;  // whole wave leaves together
-    float acc[MMAX];
+    const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CPW;
+    if (n0 >= p.N) return;  // whole wave leaves together
+    float acc[CPW][MM];
 #pragma unroll
-    for (int m = 0; m < MMAX; ++m) acc[m] = 0.0f;
-    const bf16_t* wrow = p.W + static_cast<int64_t>(n) * p.ldw;
-    for (int k = lane * 8; k < p.K; k += 512) {
-        Vec16<bf16_t> w = ld16(wrow + k);
-        float wf[8];
+    for (int c = 0; c < CPW; ++c)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) wf[e] = bf2f(w.v[e]);
+        for (int m = 0; m < MM; ++m) acc[c][m] = 0.0f;
+    const bf16_t* wrow[CPW];
 #pragma unroll
-        for (int m = 0; m < MMAX; ++m) {
-            if (m < p.M) {
-                Vec16<bf16_t> a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
+    for (int c = 0; c < CPW; ++c) wrow[c] = p.W + static_cast<int64_t>(n0 + c < p.N ? n0 + c : n0) * p.ldw;
+    for (int k0 = lane * 8; k0 < p.K; k0 += 512 * U) {
+        Vec16<bf16_t> w[U][CPW];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[m] += wf[e] * bf2f(a.v[e]);
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + u * 512;
+            // past the end: a harmless re-read, skipped below
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) w[u][c] = ld16(wrow[c] + (k < p.K ? k : k0));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + u * 512;
+            if (k >= p.K) break;
+            float af[MM][8];
+#pragma unroll
+            for (int m = 0; m < MM; ++m) {
+                const Vec16<bf16_t> a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) af[m][e] = bf2f(a.v[e]);
             }
+#pragma unroll
+            for (int c = 0; c < CPW; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float wf = bf2f(w[u][c].v[e]);
+#pragma unroll
+                    for (int m = 0; m < MM; ++m) acc[c][m] += wf * af[m][e];
+                }
         }
     }
 #pragma unroll
-    for (int m = 0; m < MMAX; ++m) acc[m] = group_sum<64>(acc[m]);
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+        for (int m = 0; m < MM; ++m) acc[c][m] = group_sum<64>(acc[c][m]);
     if (lane == 0) {
-        const float b = p.bias ? bf2f(p.bias[n]) : 0.0f;
-        for (int m = 0; m < p.M && m < MMAX; ++m) {
-            float t = acc[m] + b;
-            if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
-            t = bf2f(f2bf(t));
-            if (p.gate != nullptr) {
-                const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
-                const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
-                t = r + bf2f(f2bf(g * t));
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) {
+            const int n = n0 + c;
+            if (n >= p.N) break;
+            const float b = p.bias ? bf2f(p.bias[n]) : 0.0f;
+#pragma unroll
+            for (int m = 0; m < MM; ++m) {
+                float t = acc[c][m] + b;
+                if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
+                t = bf2f(f2bf(t));
+                if (p.gate != nullptr) {
+                    const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
+                    const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
+                    t = r + bf2f(f2bf(g * t));
+                }
+                bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
+                                            : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
+                *dst = f2bf(t);
             }
-            bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
-                                        : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
-            *dst = f2bf(t);
         }
     }
+}
+
+template <int MM>
+static void launch_gemv(const GemmParams& p, hipStream_t st) {
+    const unsigned grid = (unsigned)((p.N + 4 * kGemvCols - 1) / (4 * kGemvCols));
+    hipLaunchKernelGGL((gemv_small_m_kernel<MM>), dim3(grid), dim3(256), 0, st, p);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -674,7 +712,16 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
         return check_launch("flux_linear_bf16");
     }
     if (p.M <= 8) {
-        hipLaunchKernelGGL((gemv_small_m_kernel<8>), dim3((unsigned)((p.N + 3) / 4)), dim3(256), 0, st, p);
+        switch (p.M) {
+            case 1: launch_gemv<1>(p, st); break;
+            case 2: launch_gemv<2>(p, st); break;
+            case 3: launch_gemv<3>(p, st); break;
+            case 4: launch_gemv<4>(p, st); break;
+            case 5: launch_gemv<5>(p, st); break;
+            case 6: launch_gemv<6>(p, st); break;
+            case 7: launch_gemv<7>(p, st); break;
+            default: launch_gemv<8>(p, st); break;
+        }
         return check_launch("flux_linear_bf16");
     }
     // 256 x 256 tiles once they fill most of the 256 CUs; below that 128 x 128 tiles (two workgroups
