@@ -44,6 +44,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run plain device-to-device copies of 256 MiB (reference for scaling FETCH_SIZE / "
+                         "WRITE_SIZE counter readings), then exit")
     return ap.parse_args()
 
 
@@ -92,6 +95,16 @@ def kernel_table(torch):
             ach, peak, unit = work / us / 1e6, MFMA_PEAK_TFLOPS, "TFLOP/s"
         out[name] = {"us": round(us, 2), "bound": bound, "achieved": round(ach, 1), "unit": unit,
                      "frac": round(ach / peak, 4), "work": work, **({"note": note} if note else {})}
+
+    # What a plain device-to-device copy reaches at the sizes of the row-wise kernels below (the
+    # practical HBM ceiling of this machine for read-once / write-once traffic, launch included).
+    for mb in (27, 81):
+        n = mb * 1024 * 1024 // 2
+        sets = [(torch.empty(n, dtype=torch.bfloat16, device=dev).normal_(), torch.empty(n, dtype=torch.bfloat16, device=dev))
+                for _ in range(n_sets(4 * n))]
+        launches = [(lambda a=a, y=y: y.copy_(a)) for a, y in sets]
+        entry(f"copy_{mb}MiB_reference", _time_launches(torch, launches), "hbm", 4 * n, "torch copy_ (device-to-device), same rotation")
+        del sets, launches
 
     # C1: QK RMSNorm, x [1,24,4608,128]
     x, w = cfg.config1(dev)
@@ -220,6 +233,16 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.calibrate_copy:
+        n = 256 * 1024 * 1024
+        srcs = [torch.full((n,), i, dtype=torch.uint8, device=dev) for i in range(4)]
+        dst = torch.empty(n, dtype=torch.uint8, device=dev)
+        for a in srcs * 2:
+            dst.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "8 device-to-device copies", "bytes_read_per_copy": n, "bytes_written_per_copy": n}))
+        return
+
     x, vec, pe, sd = cfg.config5_block(dev)
     blk = tk.SingleStreamBlock(3072, 24).to(torch.bfloat16).to(dev)
     blk.load_state_dict(sd)
@@ -278,7 +301,7 @@ def main():
         "block_tflops": round(BLOCK_GFLOP / ms_per_step, 1),
         "block_frac_of_mfma_peak": round(BLOCK_GFLOP / ms_per_step / MFMA_PEAK_TFLOPS, 4),
         "roofline": {
-            "kernel": "gemm_nt_kernel (linear1: 4608 x 21504 x 3072, bias, split qkv / GELU(mlp) epilogue)",
+            "kernel": "gemm_nt_ring_kernel<4> (linear1: 4608 x 21504 x 3072, bias, split qkv / GELU(mlp) epilogue)",
             "bound": "mfma", "achieved": round(l1_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(l1_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": LINEAR1_TRAFFIC_BYTES,
             "launch_us": round(l1_us, 1), "launches_timed": len(l1_events),
