@@ -31,10 +31,11 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 BLOCK_GFLOP = 1304.65       # linear1 + attention + linear2 + modulation projection
 LINEAR1_FLOP = 2.0 * 4608 * 21504 * 3072
 
-# HBM traffic of one linear1 launch, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs
-# (KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size.
-# None until such a pair of runs has been summarised under profiles/.
-LINEAR1_TRAFFIC_BYTES = None
+# Fabric-side traffic of one linear1 launch (what the L2s fetch from / write to Infinity Cache + HBM),
+# from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script, each scaled by what
+# the same counter reads for a plain 256 MiB copy (`--calibrate-copy`): fetch 505970.8 x 2.000 KiB,
+# write 193536.0 x 1.000 KiB per dispatch. The summary is profiles/gemm_linear1_linear2_4608_hbm_traffic.md.
+LINEAR1_TRAFFIC_BYTES = int((505970.8 * 2.000 + 193536.0 * 1.000) * 1024)
 
 
 def parse_args():
