@@ -366,8 +366,12 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// Multiplies K slabs [kb, ke) of the tile at (m0, n0) into acc (cleared first). On return every
+// buffer load of the wave has landed and all waves have passed a barrier, so the ring may be
+// reused (the epilogue parks its bf16 blocks there).
 template <int MI>
-__global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p) {
+__device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, int m0, int n0, int kb, int ke,
+                                                f32x16 (&acc)[MI][MI]) {
     constexpr int NJ = MI;
     constexpr int BM = 64 * MI, BN = BM, BK = 64;
     constexpr int ROWB = BK * 2, KSUB = BK / 16;
@@ -382,12 +386,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     constexpr int EARLY = NL - (GB + 1) / 2;     // loads of a group issued behind the previous slab's barrier
     static_assert(MFMAS % READS == 0 && KSUB == 4 && NSLOT == 2 * NL, "schedule shape");
     static_assert(4 * WROWS * WCOLS * 2 <= NU * UNIT, "epilogue tile must fit the ring");
-    __shared__ __attribute__((aligned(1024))) char lds[NU * UNIT];
-
-    int tm, tn;
-    if (!tile_of_block(p, tm, tn)) return;
-    const int m0 = tm * BM, n0 = tn * BN;
-
+    (void)BN; (void)WCOLS;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -410,10 +409,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
         voff_a[i] = r < rows_a ? static_cast<uint32_t>((r * p.lda + lchunk * 8) * 2) : kOutOfRange;
         voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
     }
-    const int nk = (p.K + BK - 1) / BK;
+    // the slab range ends at ke: everything from there on reads as zeros, like the K tail
+    const int k_end = min(p.K, ke * BK);
     // Slabs past the end and the part of the last slab past K read as zeros: both are "this
     // thread's chunk starts at or past K" (K is a multiple of 8, so a chunk is all in or all out).
-    auto slab_mask = [&](int kt) -> uint32_t { return kt * BK + lchunk * 8 >= p.K ? kOutOfRange : 0u; };
+    auto slab_mask = [&](int kt) -> uint32_t { return kt * BK + lchunk * 8 >= k_end ? kOutOfRange : 0u; };
     // ring offsets are wave-uniform byte offsets of a unit inside the ring
     auto load_a = [&](int uoff, int pass, int kt, uint32_t mask) {
         load_chunk(rsrc_a, lds + uoff + pass * 4096 + wave * 1024, voff_a[pass] | mask, kt * ROWB);
@@ -437,7 +437,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
         koff_w[kk] = (wn * WCOLS + frow) * ROWB + ko;
     }
 
-    f32x16 acc[MI][NJ];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -498,15 +497,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
 
     // Prologue: slab 0, A(1) and the first loads of G(0); slab 0 must have landed, the rest flies on.
     {
-        const uint32_t k0 = slab_mask(0), k1 = slab_mask(1);
+        const uint32_t k0 = slab_mask(kb), k1 = slab_mask(kb + 1);
 #pragma unroll
-        for (int i = 0; i < PU; ++i) load_a(0, i, 0, k0);
+        for (int i = 0; i < PU; ++i) load_a(0, i, kb, k0);
 #pragma unroll
-        for (int i = 0; i < PU; ++i) load_w(UNIT, i, 0, k0);
+        for (int i = 0; i < PU; ++i) load_w(UNIT, i, kb, k0);
 #pragma unroll
-        for (int i = 0; i < PU; ++i) load_a(2 * UNIT, i, 1, k1);
+        for (int i = 0; i < PU; ++i) load_a(2 * UNIT, i, kb + 1, k1);
 #pragma unroll
-        for (int i = 0; i < EARLY; ++i) load_w(3 * UNIT, i, 1, k1);
+        for (int i = 0; i < EARLY; ++i) load_w(3 * UNIT, i, kb + 1, k1);
         wait_loads_and_barrier<PU + EARLY>();
 #pragma unroll
         for (int r = 0; r < READS; ++r) read_frag(0, 0, UNIT, 0, r);
@@ -516,8 +515,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
 
     {
         int ua = 0, uw = UNIT, ua1 = 2 * UNIT, uw1 = 3 * UNIT, ua2 = 4 * UNIT;
-        uint32_t m1 = slab_mask(1), m2 = slab_mask(2);
-        for (int kt = 0; kt < nk; ++kt) {
+        uint32_t m1 = slab_mask(kb + 1), m2 = slab_mask(kb + 2);
+        for (int kt = kb; kt < ke; ++kt) {
             uint32_t m3;
             slab(kt, ua, uw, ua1, uw1, ua2, m1, m2, m3);
             // the ring advances by two units
@@ -530,7 +529,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     // retire them before the epilogue reuses the ring.
     wait_vmem_all();
     __syncthreads();
-    gemm_epilogue<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+}
+
+
+template <int MI>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p) {
+    constexpr int BM = 64 * MI, BK = 64, NU = 5, UNIT = BM * BK * 2;
+    __shared__ __attribute__((aligned(1024))) char lds[NU * UNIT];
+    int tm, tn;
+    if (!tile_of_block(p, tm, tn)) return;
+    const int m0 = tm * BM, n0 = tn * BM;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    f32x16 acc[MI][MI];
+    gemm_tile_slabs<MI>(p, lds, m0, n0, 0, (p.K + BK - 1) / BK, acc);
+    gemm_epilogue<MI, MI>(p, acc, lds, m0, n0, wave, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
