@@ -76,7 +76,7 @@ __device__ __forceinline__ void lds_load16_raw(u32x4 rsrc, uint32_t lds_addr, ui
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
-                 : "memory", "m0");
+                 : "memory");  // m0 is written; nothing else in this file's kernel reads it (LDS ops need no m0 on gfx9+)
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p));
