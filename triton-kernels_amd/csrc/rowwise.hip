@@ -261,62 +261,69 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_block(
 // For bf16 storage the normalised value, (1+scale) and the product are each rounded to bf16 before
 // the next step, the evaluation order of functional/normalization.py:6-12 on bf16 tensors.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int G, int ITER>
+// Straight-line: rows past the end and columns past n are clamped for the loads (x, scale and shift
+// vectors all go out before the first reduction) and masked in the sums; only the stores are
+// predicated. FULL = the row fills the lanes exactly (n == G * ITER * VEC), no column masks at all.
+template <typename T, int G, int ITER, bool FULL>
 __global__ __launch_bounds__(kBlock) void ln_mod_fwd_regs(
     const T* __restrict__ x, const T* __restrict__ scale, const T* __restrict__ shift, T* __restrict__ y,
     int64_t rows, int64_t seq, int n, int64_t mod_stride, float eps) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int ROWS_PER_BLOCK = kBlock / G;
     const int lane = threadIdx.x % G;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / G;
-    const bool row_ok = row < rows;
+    const int64_t row_raw = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / G;
+    const bool row_ok = row_raw < rows;
+    const int64_t row = row_ok ? row_raw : rows - 1;
+    const int64_t b = row / seq;
+    const T* xr = x + row * n;
+    const T* sc = scale + b * mod_stride;
+    const T* sh = shift + b * mod_stride;
 
-    RowRegs<T, G, ITER> r;
-    r.load(x + (row_ok ? row : 0) * n, lane, n, row_ok);
-
+    Vec16<T> xv[ITER], av[ITER], dv[ITER];
+    bool in[ITER];
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int c = (it * G + lane) * VEC;
+        in[it] = FULL || c < n;
+        const int cl = in[it] ? c : 0;
+        xv[it] = ld16(xr + cl);
+        av[it] = ld16(sc + cl);
+        dv[it] = ld16(sh + cl);
+    }
+    float xf[ITER][VEC];
     float s = 0.0f;
 #pragma unroll
     for (int it = 0; it < ITER; ++it)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) s += r.x[it][e];
+        for (int e = 0; e < VEC; ++e) {
+            xf[it][e] = in[it] ? Elem<T>::load(xv[it].v[e]) : 0.0f;
+            s += xf[it][e];
+        }
     s = group_sum<G>(s);
     const float mean = s / static_cast<float>(n);
     float q = 0.0f;
 #pragma unroll
-    for (int it = 0; it < ITER; ++it) {
-        int c = (it * G + lane) * VEC;
-        if (c < n) {
+    for (int it = 0; it < ITER; ++it)
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                float d = r.x[it][e] - mean;
-                q += d * d;
-            }
+        for (int e = 0; e < VEC; ++e) {
+            const float d = in[it] ? xf[it][e] - mean : 0.0f;
+            q += d * d;
         }
-    }
     q = group_sum<G>(q);
     const float rstd = rsqrtf(q / static_cast<float>(n) + eps);
 
-    if (!row_ok) return;
-    const int64_t b = row / seq;
-    const T* sc = scale + b * mod_stride;
-    const T* sh = shift + b * mod_stride;
     T* yrow = y + row * n;
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
-        int c = (it * G + lane) * VEC;
-        if (c < n) {
-            float a[VEC], d[VEC];
-            load_vecf<T, VEC>(sc + c, a);
-            load_vecf<T, VEC>(sh + c, d);
-            Vec16<T> o;
+        const int c = (it * G + lane) * VEC;
+        Vec16<T> o;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                float nv = Elem<T>::round((r.x[it][e] - mean) * rstd);
-                float g = Elem<T>::round(1.0f + a[e]);
-                o.v[e] = Elem<T>::store(Elem<T>::round(nv * g) + d[e]);
-            }
-            st16(yrow + c, o);
+        for (int e = 0; e < VEC; ++e) {
+            const float nv = Elem<T>::round((xf[it][e] - mean) * rstd);
+            const float g = Elem<T>::round(1.0f + Elem<T>::load(av[it].v[e]));
+            o.v[e] = Elem<T>::store(Elem<T>::round(nv * g) + Elem<T>::load(dv[it].v[e]));
         }
+        if (row_ok && in[it]) st16(yrow + c, o);
     }
 }
 
@@ -450,8 +457,13 @@ static int ln_mod_launch(const void* x, const void* scale, const void* shift, vo
     const bool vec_ok = aligned16(x) && aligned16(y) && aligned16(scale) && aligned16(shift) && mod_stride % VEC == 0;
     if (plan.G != 0 && vec_ok) {
 #define CALL(G_, I_)                                                                                        \
-    hipLaunchKernelGGL((ln_mod_fwd_regs<T, G_, I_>), dim3((unsigned)((rows + kBlock / G_ - 1) / (kBlock / G_))),  \
-                       dim3(kBlock), 0, st, xp, scp, shp, yp, rows, seq, n, mod_stride, eps)
+    do {                                                                                                    \
+        const dim3 grid_((unsigned)((rows + kBlock / G_ - 1) / (kBlock / G_)));                              \
+        if (n == G_ * I_ * VEC)                                                                             \
+            hipLaunchKernelGGL((ln_mod_fwd_regs<T, G_, I_, true>), grid_, dim3(kBlock), 0, st, xp, scp, shp, yp, rows, seq, n, mod_stride, eps);  \
+        else                                                                                                \
+            hipLaunchKernelGGL((ln_mod_fwd_regs<T, G_, I_, false>), grid_, dim3(kBlock), 0, st, xp, scp, shp, yp, rows, seq, n, mod_stride, eps); \
+    } while (0)
         FLUX_DISPATCH_GI(plan, CALL);
 #undef CALL
     } else {
