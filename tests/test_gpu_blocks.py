@@ -58,7 +58,13 @@ def test_double_stream_block(batch_size, img_seq_len):
     pe = randn(g, 1, 1, txt_len + img_seq_len, HEAD_DIM // 2, 2, 2).to(DEV)
     with torch.no_grad():
         r_img, r_txt = ref(img=img, txt=txt, vec=vec, pe=pe)
-        h_img, h_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
+        h_img, h_txt = hip(img=img, txt=txt, vec=vec, pe=pe)         # fused, txt chain on a side stream
+        for _ in range(3):                                           # the two streams join correctly every time
+            a_img, a_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
+            assert torch.equal(a_img, h_img) and torch.equal(a_txt, h_txt)
+        hip.two_streams = False
+        s_img, s_txt = hip(img=img, txt=txt, vec=vec, pe=pe)         # fused, one stream: same kernels, same bits
+        assert torch.equal(s_img, h_img) and torch.equal(s_txt, h_txt)
         hip.fused = False
         u_img, u_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
     torch.testing.assert_close(h_img, r_img, atol=0.1, rtol=0)
