@@ -379,8 +379,8 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
                 constexpr int kb = u / 8, r = (u % 8) * 2;
                 // The empty asm ties the unit's inputs to this slot: without it the optimiser is free
                 // to hoist all the (mutually independent) exponentials into one clump.
-                float a0 = s_cur[qb][kb][r], a1 = s_cur[qb][kb][r + 1];
-                asm volatile("" : "+v"(a0), "+v"(a1));
+                asm volatile("" : "+v"(s_cur[qb][kb]));
+                const float a0 = s_cur[qb][kb][r], a1 = s_cur[qb][kb][r + 1];
                 const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a0, c, -mc[qb]));
                 const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a1, c, -mc[qb]));
                 pw[qb][u] = pack2_bf16(p0, p1);
