@@ -28,13 +28,16 @@ struct PrepParams {
     int scale_vec;  // 1: every RMS scale pointer is 16-byte aligned (vector loads)
 };
 
-// Row of source s at (b, h, pos): txt rows first, then img rows. Both candidates are formed and one
-// is selected, so there is no branch in front of the load.
+// Row of source s at (b, h0, pos) and the element stride from one head to the next: txt rows first,
+// then img rows. Both candidates are formed and one is selected, so there is no branch in front of
+// the loads, and the per-head addresses are one multiply-add away.
 template <typename T>
-__device__ __forceinline__ const T* src_row(const Src& s, int64_t b, int64_t h, int64_t pos, int64_t Lt) {
-    const T* t = static_cast<const T*>(s.txt) + b * s.t_sb + h * s.t_sh + pos * s.t_sl;
-    const T* i = static_cast<const T*>(s.img) + b * s.i_sb + h * s.i_sh + (pos - Lt) * s.i_sl;
-    return pos < Lt ? t : i;
+__device__ __forceinline__ const T* src_row0(const Src& s, int64_t b, int64_t h0, int64_t pos, int64_t Lt, int64_t& head_stride) {
+    const bool is_txt = pos < Lt;
+    const T* t = static_cast<const T*>(s.txt) + b * s.t_sb + h0 * s.t_sh + pos * s.t_sl;
+    const T* i = static_cast<const T*>(s.img) + b * s.i_sb + h0 * s.i_sh + (pos - Lt) * s.i_sl;
+    head_stride = is_txt ? s.t_sh : s.i_sh;
+    return is_txt ? t : i;
 }
 
 // Heads one thread walks with the same pe / scale registers: the rotation table is read once per
@@ -63,13 +66,15 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
     const bool ok = pos_raw < p.L;
     const int64_t pos = ok ? pos_raw : p.L - 1;
     const bool is_txt = pos < p.Lt;
-    int64_t hh[HG];
+    int hd[HG];      // head offset from h0, clamped to the last head
     bool hok[HG];
 #pragma unroll
     for (int g = 0; g < HG; ++g) {
         hok[g] = ok && h0 + g < p.H;
-        hh[g] = h0 + g < p.H ? h0 + g : p.H - 1;
+        hd[g] = h0 + g < p.H ? g : static_cast<int>(p.H - 1 - h0);
     }
+    const int64_t out_row0 = ((b * p.H + h0) * p.L + pos) * D;   // output row of head h0; the next head is L * D further
+    const int64_t out_head = p.L * D;
 
     // pe[pos, pair, a, j]: the lane's vector at column c covers pairs c/2 .. c/2 + VEC/2 - 1
     float f[ITER][VEC * 2];
@@ -89,16 +94,18 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
 
     // v: bit-exact copy
     if (p.v.out != nullptr) {
+        int64_t v_hs;
+        const T* v_src0 = src_row0<T>(p.v, b, h0, pos, p.Lt, v_hs);
         Vec16<T> vv[HG][ITER];
 #pragma unroll
         for (int g = 0; g < HG; ++g) {
-            const T* src = src_row<T>(p.v, b, hh[g], pos, p.Lt);
+            const T* src = v_src0 + hd[g] * v_hs;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) vv[g][it] = ld16(src + (it * G + lane) * VEC);
         }
 #pragma unroll
         for (int g = 0; g < HG; ++g) {
-            T* out = static_cast<T*>(p.v.out) + ((b * p.H + hh[g]) * p.L + pos) * D;
+            T* out = static_cast<T*>(p.v.out) + out_row0 + hd[g] * out_head;
             if (hok[g]) {
 #pragma unroll
                 for (int it = 0; it < ITER; ++it) st16(out + (it * G + lane) * VEC, vv[g][it]);
@@ -113,9 +120,11 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
     for (int which = 0; which < 2; ++which) {
         const Src& s = which == 0 ? p.q : p.k;
         if (s.out == nullptr) continue;  // uniform over the grid
+        int64_t hs;
+        const T* src0 = src_row0<T>(s, b, h0, pos, p.Lt, hs);
 #pragma unroll
         for (int g = 0; g < HG; ++g) {
-            const T* src = src_row<T>(s, b, hh[g], pos, p.Lt);
+            const T* src = src0 + hd[g] * hs;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) raw[which][g][it] = ld16(src + (it * G + lane) * VEC);
         }
@@ -145,7 +154,7 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
         if (s.out == nullptr) continue;
 #pragma unroll
         for (int g = 0; g < HG; ++g) {
-            T* out = static_cast<T*>(s.out) + ((b * p.H + hh[g]) * p.L + pos) * D;
+            T* out = static_cast<T*>(s.out) + out_row0 + hd[g] * out_head;
             if (!NORM && !ROPE) {
                 if (hok[g]) {
 #pragma unroll
