@@ -163,15 +163,17 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_block(
 // ------------------------------------------------------------------------------------------------
 // RMSNorm backward: dx = rstd*(dy*w) - rstd^3/n * sum(dy*w*x) * x ;  dscale += sum_rows dy*x*rstd.
 // One group of G lanes per row (register-resident); each block reduces its rows' dscale partials in
-// registers while walking a strip of rows per group, folds them in LDS and finishes with one atomic
-// per column per block.
+// registers while its groups walk the block's rows, folds them in LDS and finishes with one atomic
+// per column per block. All blocks finish together and their atomics land on the few cache lines of
+// dscale, where they are served one at a time: short rows (one vector per lane) therefore run as
+// 256 blocks of 1024 threads rather than 1024 blocks of 256.
 // ------------------------------------------------------------------------------------------------
-template <typename T, typename TS, int G, int ITER>
-__global__ __launch_bounds__(kBlock) void rms_norm_bwd_regs(
+template <typename T, typename TS, int G, int ITER, int BLK>
+__global__ __launch_bounds__(BLK) void rms_norm_bwd_regs(
     const T* __restrict__ dy, const T* __restrict__ x, const TS* __restrict__ scale, const float* __restrict__ rstd_in,
     T* __restrict__ dx, float* __restrict__ dscale, int64_t rows, int n, int rows_per_group) {
     constexpr int VEC = Elem<T>::VEC;
-    constexpr int GROUPS = kBlock / G;
+    constexpr int GROUPS = BLK / G;
     const int lane = threadIdx.x % G;
     const int grp = threadIdx.x / G;
 
@@ -185,33 +187,47 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_regs(
         if (c < n) load_vecf<TS, VEC>(scale + c, w[it]);
     }
 
-    const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * GROUPS + grp) * rows_per_group;
-    for (int i = 0; i < rows_per_group; ++i) {
-        const int64_t row = row0 + i;
-        const bool row_ok = row < rows;  // uniform over the group; DPP lanes of other groups unaffected
-        RowRegs<T, G, ITER> rx, rdy;
-        rx.load(x + row * n, lane, n, row_ok);
-        rdy.load(dy + row * n, lane, n, row_ok);
-        const float rstd = row_ok ? rstd_in[row] : 0.0f;
-        float dot = 0.0f;
+    // A block owns GROUPS * rows_per_group consecutive rows and its groups take them interleaved, so
+    // one step of the block reads a contiguous span; U rows per group are requested before the first
+    // is used.
+    constexpr int U = ITER == 1 ? 4 : (ITER == 2 ? 2 : 1);
+    const int64_t block_row0 = static_cast<int64_t>(blockIdx.x) * GROUPS * rows_per_group;
+    for (int i0 = 0; i0 < rows_per_group; i0 += U) {
+        RowRegs<T, G, ITER> rx[U], rdy[U];
+        float rstd[U];
+        bool ok[U];
+        int64_t row[U];
 #pragma unroll
-        for (int it = 0; it < ITER; ++it)
+        for (int u = 0; u < U; ++u) {
+            row[u] = block_row0 + static_cast<int64_t>(i0 + u) * GROUPS + grp;
+            ok[u] = i0 + u < rows_per_group && row[u] < rows;  // uniform over the group
+            const int64_t r = ok[u] ? row[u] : 0;
+            rx[u].load(x + r * n, lane, n, ok[u]);
+            rdy[u].load(dy + r * n, lane, n, ok[u]);
+            rstd[u] = ok[u] ? rstd_in[r] : 0.0f;
+        }
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) dot += rdy.x[it][e] * w[it][e] * rx.x[it][e];
-        dot = group_sum<G>(dot);
-        const float coef = -rstd * rstd * rstd * dot / static_cast<float>(n);
-        if (row_ok) {
+        for (int u = 0; u < U; ++u) {
+            float dot = 0.0f;
 #pragma unroll
-            for (int it = 0; it < ITER; ++it) {
-                int c = (it * G + lane) * VEC;
-                if (c < n) {
-                    Vec16<T> o;
+            for (int it = 0; it < ITER; ++it)
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        o.v[e] = Elem<T>::store(rstd * rdy.x[it][e] * w[it][e] + coef * rx.x[it][e]);
-                        dw[it][e] += rdy.x[it][e] * rx.x[it][e] * rstd;
+                for (int e = 0; e < VEC; ++e) dot += rdy[u].x[it][e] * w[it][e] * rx[u].x[it][e];
+            dot = group_sum<G>(dot);
+            const float coef = -rstd[u] * rstd[u] * rstd[u] * dot / static_cast<float>(n);
+            if (ok[u]) {
+#pragma unroll
+                for (int it = 0; it < ITER; ++it) {
+                    int c = (it * G + lane) * VEC;
+                    if (c < n) {
+                        Vec16<T> o;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            o.v[e] = Elem<T>::store(rstd[u] * rdy[u].x[it][e] * w[it][e] + coef * rx[u].x[it][e]);
+                            dw[it][e] += rdy[u].x[it][e] * rx[u].x[it][e] * rstd[u];
+                        }
+                        st16(dx + row[u] * n + c, o);
                     }
-                    st16(dx + row * n + c, o);
                 }
             }
         }
@@ -226,7 +242,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_regs(
         for (int e = 0; e < VEC; ++e) dw_lds[grp * COLS + c + e] = dw[it][e];
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < n; c += kBlock) {
+    for (int c = threadIdx.x; c < n; c += BLK) {
         float t = 0.0f;
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) t += dw_lds[g * COLS + c];
@@ -424,17 +440,19 @@ static int rms_bwd_launch(const void* dy, const void* x, const void* scale, cons
     RowPlan plan = plan_row(n, VEC);
     const bool vec_ok = aligned16(dy) && aligned16(x) && aligned16(dx) && (sizeof(TS) * VEC != 16 || aligned16(scale));
     if (plan.G != 0 && plan.ITER <= 4 && vec_ok) {
-        // Enough groups to fill the chip, each walking a strip of rows so that dscale sees few atomics.
-        const int groups_per_block = kBlock / plan.G;
-        const size_t lds_bytes = sizeof(float) * kBlock * plan.ITER * VEC;
-        int64_t want_groups = 1024LL * groups_per_block;
-        int rows_per_group = (int)((rows + want_groups - 1) / want_groups);
-        if (rows_per_group < 1) rows_per_group = 1;
-        int64_t ngroups = (rows + rows_per_group - 1) / rows_per_group;
-        unsigned grid = (unsigned)((ngroups + groups_per_block - 1) / groups_per_block);
-#define CALL(G_, I_)                                                                                            \
-    hipLaunchKernelGGL((rms_norm_bwd_regs<T, TS, G_, (I_ > 4 ? 4 : I_)>), dim3(grid), dim3(kBlock), lds_bytes, st, dyp, xp, \
-                       sp, rstd, dxp, dscale, rows, n, rows_per_group)
+#define CALL(G_, I_)                                                                                         \
+    do {                                                                                                     \
+        constexpr int IT = (I_ > 4 ? 4 : I_);                                                                \
+        constexpr int BLK = IT == 1 ? 1024 : kBlock;                                                         \
+        constexpr int GROUPS = BLK / G_;                                                                     \
+        const int64_t want_blocks = IT == 1 ? 256 : 1024;  /* few blocks: few atomics on dscale */           \
+        int64_t rpg = (rows + want_blocks * GROUPS - 1) / (want_blocks * GROUPS);                            \
+        if (rpg < 1) rpg = 1;                                                                                \
+        const unsigned grid = (unsigned)((rows + rpg * GROUPS - 1) / (rpg * GROUPS));                        \
+        const size_t lds_bytes = sizeof(float) * BLK * IT * VEC;                                             \
+        hipLaunchKernelGGL((rms_norm_bwd_regs<T, TS, G_, IT, BLK>), dim3(grid), dim3(BLK), lds_bytes, st, dyp, xp, sp, \
+                           rstd, dxp, dscale, rows, n, (int)rpg);                                            \
+    } while (0)
         FLUX_DISPATCH_GI(plan, CALL);
 #undef CALL
     } else {
