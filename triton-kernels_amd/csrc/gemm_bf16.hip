@@ -23,7 +23,7 @@
 namespace flux {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
@@ -105,48 +105,45 @@ __device__ __forceinline__ float tanh_gelu_fast(float x) {
 }
 
 template <int MI, int NJ>
-__device__ __forceinline__ void gemm_epilogue_checked(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+__device__ __forceinline__ void gemm_epilogue_checked(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
                                                    int wave, int lane) {
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
     constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;  // bytes per row, 16-byte chunks per row
     constexpr int RPI = 64 / C_CH;                         // rows one wave-wide 16-byte access covers
+    constexpr int NQ = 2 * NJ;                             // column quads of a lane: one per 16-column fragment
     const int wm = wave >> 1, wn = wave & 1;
-    const int frow = lane & 31, fhalf = lane >> 5;
+    const int frow = lane & 15, fq = lane >> 4;            // accumulator: row frow of a 16-row fragment, columns fq*4..+3
     char* cw = lds + wave * (WROWS * C_PITCH);
     const int wave_n0 = n0 + wn * WCOLS;
     const int wave_m0 = m0 + wm * WROWS;
 
-    // bias for the lane's 4*NJ column quads
-    float bv[NJ][4][4];
+    // bias for the lane's NQ column quads
+    float bv[NQ][4];
     const bool bias_fast = p.bias != nullptr && p.bias_vec;
     if (bias_fast) {
         const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + j * 32 + g * 8 + fhalf * 4) * 2, 0, 0);
-                bv[j][g][0] = __uint_as_float(raw.x << 16);
-                bv[j][g][1] = __uint_as_float(raw.x & 0xffff0000u);
-                bv[j][g][2] = __uint_as_float(raw.y << 16);
-                bv[j][g][3] = __uint_as_float(raw.y & 0xffff0000u);
-            }
+        for (int q = 0; q < NQ; ++q) {
+            const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + q * 16 + fq * 4) * 2, 0, 0);
+            bv[q][0] = __uint_as_float(raw.x << 16);
+            bv[q][1] = __uint_as_float(raw.x & 0xffff0000u);
+            bv[q][2] = __uint_as_float(raw.y << 16);
+            bv[q][3] = __uint_as_float(raw.y & 0xffff0000u);
+        }
     } else {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int q = 0; q < NQ; ++q)
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int n = wave_n0 + j * 32 + g * 8 + fhalf * 4 + e;
-                    bv[j][g][e] = (p.bias != nullptr && n < p.N) ? bf2f(p.bias[n]) : 0.0f;
-                }
+            for (int e = 0; e < 4; ++e) {
+                const int n = wave_n0 + q * 16 + fq * 4 + e;
+                bv[q][e] = (p.bias != nullptr && n < p.N) ? bf2f(p.bias[n]) : 0.0f;
+            }
     }
 
-    // LDS write address of column quad (j, g) in this lane's row, without the 32-row block offset
-    int waddr[NJ * 4];
+    // LDS write address of column quad q in this lane's row, without the 16-row fragment offset
+    int waddr[NQ];
 #pragma unroll
-    for (int c = 0; c < NJ * 4; ++c) waddr[c] = frow * C_PITCH + ((c ^ (frow & (C_CH - 1))) * 16) + fhalf * 8;
+    for (int q = 0; q < NQ; ++q) waddr[q] = frow * C_PITCH + (((q * 2 + (fq >> 1)) ^ (frow & (C_CH - 1))) * 16) + (fq & 1) * 8;
     // read side: lane -> (row within the pass = lane / C_CH, chunk = lane % C_CH)
     const int rrow = lane / C_CH, rch = lane % C_CH;
 
@@ -154,23 +151,23 @@ __device__ __forceinline__ void gemm_epilogue_checked(const GemmParams& p, f32x1
     const bool gelu_some = p.act == FLUX_ACT_GELU_TANH && !gelu_all && wave_n0 + WCOLS > p.act_begin;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
-        // ---- accumulators of block row i -> bf16 -> LDS
+        // ---- accumulators of block row i (two 16-row fragments) -> bf16 -> LDS
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int q = 0; q < NQ; ++q) {
                 float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e] + bv[j][g][e];
+                for (int e = 0; e < 4; ++e) v[e] = acc[2 * i + t][q][e] + bv[q][e];
                 if (gelu_all) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = tanh_gelu_fast(v[e]);
                 } else if (gelu_some) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (wave_n0 + j * 32 + g * 8 + fhalf * 4 + e >= p.act_begin) v[e] = tanh_gelu_fast(v[e]);
+                        if (wave_n0 + q * 16 + fq * 4 + e >= p.act_begin) v[e] = tanh_gelu_fast(v[e]);
                 }
-                *reinterpret_cast<u32x2*>(cw + i * 32 * C_PITCH + waddr[j * 4 + g]) = pack4_bf16(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<u32x2*>(cw + (i * 32 + t * 16) * C_PITCH + waddr[q]) = pack4_bf16(v[0], v[1], v[2], v[3]);
             }
         __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
 
@@ -219,43 +216,40 @@ __device__ __forceinline__ void gemm_epilogue_checked(const GemmParams& p, f32x1
 // Everything lane-dependent is computed once; per store only a wave-uniform row offset changes, so
 // the stores use a scalar base plus a 32-bit lane offset.
 template <int MI, int NJ, bool GELU, bool GATE>
-__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
                                                    int wave, int lane) {
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
     constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;
     constexpr int RPI = 64 / C_CH;      // rows per wave-wide 16-byte access
     constexpr int NIT = 32 / RPI;       // accesses per 32-row block
+    constexpr int NQ = 2 * NJ;          // column quads of a lane: one per 16-column fragment
     const int wm = wave >> 1, wn = wave & 1;
-    const int frow = lane & 31, fhalf = lane >> 5;
+    const int frow = lane & 15, fq = lane >> 4;
     char* cw = lds + wave * (WROWS * C_PITCH);
     const int wave_n0 = n0 + wn * WCOLS;
     const int wave_m0 = m0 + wm * WROWS;
 
-    float bv[NJ][4][4];
+    float bv[NQ][4];
     if (p.bias != nullptr) {
         const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + j * 32 + g * 8 + fhalf * 4) * 2, 0, 0);
-                bv[j][g][0] = __uint_as_float(raw.x << 16);
-                bv[j][g][1] = __uint_as_float(raw.x & 0xffff0000u);
-                bv[j][g][2] = __uint_as_float(raw.y << 16);
-                bv[j][g][3] = __uint_as_float(raw.y & 0xffff0000u);
-            }
+        for (int q = 0; q < NQ; ++q) {
+            const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + q * 16 + fq * 4) * 2, 0, 0);
+            bv[q][0] = __uint_as_float(raw.x << 16);
+            bv[q][1] = __uint_as_float(raw.x & 0xffff0000u);
+            bv[q][2] = __uint_as_float(raw.y << 16);
+            bv[q][3] = __uint_as_float(raw.y & 0xffff0000u);
+        }
     } else {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int q = 0; q < NQ; ++q)
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) bv[j][g][e] = 0.0f;
+            for (int e = 0; e < 4; ++e) bv[q][e] = 0.0f;
     }
 
-    int waddr[NJ * 4];
+    int waddr[NQ];
 #pragma unroll
-    for (int c = 0; c < NJ * 4; ++c) waddr[c] = frow * C_PITCH + ((c ^ (frow & (C_CH - 1))) * 16) + fhalf * 8;
+    for (int q = 0; q < NQ; ++q) waddr[q] = frow * C_PITCH + (((q * 2 + (fq >> 1)) ^ (frow & (C_CH - 1))) * 16) + (fq & 1) * 8;
     const int rrow = lane / C_CH, rch = lane % C_CH;
     // read address for access `it` of a block: row = it*RPI + rrow; the swizzle term repeats every 16 rows
     constexpr int NSW = (16 / RPI) < NIT ? (16 / RPI) : NIT;
@@ -282,16 +276,16 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x16 (
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int q = 0; q < NQ; ++q) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    v[e] = acc[i][j][g * 4 + e] + bv[j][g][e];
+                    v[e] = acc[2 * i + t][q][e] + bv[q][e];
                     if (GELU) v[e] = tanh_gelu_fast(v[e]);
                 }
-                *reinterpret_cast<u32x2*>(cw + i * 32 * C_PITCH + waddr[j * 4 + g]) = pack4_bf16(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<u32x2*>(cw + (i * 32 + t * 16) * C_PITCH + waddr[q]) = pack4_bf16(v[0], v[1], v[2], v[3]);
             }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -318,7 +312,7 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x16 (
 }
 
 template <int MI, int NJ>
-__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[MI][NJ], char* lds, int m0, int n0,
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
                                               int wave, int lane) {
     constexpr int BM = 64 * MI, BN = 64 * NJ, WCOLS = 32 * NJ;
     const int wave_n0 = n0 + (wave & 1) * WCOLS;
@@ -371,20 +365,22 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 // reused (the epilogue parks its bf16 blocks there).
 template <int MI>
 __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, int m0, int n0, int kb, int ke,
-                                                f32x16 (&acc)[MI][MI]) {
+                                                f32x4 (&acc)[2 * MI][2 * MI]) {
     constexpr int NJ = MI;
+    constexpr int FM = 2 * MI, FN = 2 * NJ;      // 16-row fragments per wave and side
     constexpr int BM = 64 * MI, BN = BM, BK = 64;
-    constexpr int ROWB = BK * 2, KSUB = BK / 16;
+    constexpr int ROWB = BK * 2, KSUB = BK / 32;
     constexpr int UNIT = BM * ROWB, NU = 5;
     constexpr int PU = BM / 32;                  // buffer loads per thread per unit
     constexpr int NL = 2 * PU;                   // loads per group G(kt) = W(kt+1), A(kt+2)
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
-    constexpr int READS = MI + NJ, MFMAS = MI * NJ, PER = MFMAS / READS;
-    constexpr int BS = READS / 4;                // slots of step 3 in front of the barrier
+    constexpr int READS = FM + FN, MFMAS = FM * FN, PER = MFMAS / READS;
+    constexpr int BS = READS / 4;                // slots of the last step in front of the barrier
     constexpr int NSLOT = KSUB * READS;          // issue slots per slab
-    constexpr int GB = 3 * READS + BS;           // first slot behind the barrier
+    constexpr int GB = (KSUB - 1) * READS + BS;  // first slot behind the barrier
     constexpr int EARLY = NL - (GB + 1) / 2;     // loads of a group issued behind the previous slab's barrier
-    static_assert(MFMAS % READS == 0 && KSUB == 4 && NSLOT == 2 * NL, "schedule shape");
+    static_assert(MFMAS % READS == 0 && KSUB == 2 && NSLOT == 2 * NL && GB % 2 == 0, "schedule shape");
+    static_assert(2 * (NSLOT - GB) >= READS, "the next slab's first fragments are read two per slot behind the barrier");
     static_assert(4 * WROWS * WCOLS * 2 <= NU * UNIT, "epilogue tile must fit the ring");
     (void)BN; (void)WCOLS;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -428,35 +424,36 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
     };
 
     // fragment addressing
-    const int frow = lane & 31, fhalf = lane >> 5;
+    // v_mfma_f32_16x16x32_bf16 operand: lane holds row lane % 16, k = (lane / 16) * 8 .. +8 of a K=32 step
+    const int frow = lane & 15, fq = lane >> 4;
     int koff_a[KSUB], koff_w[KSUB];
 #pragma unroll
     for (int kk = 0; kk < KSUB; ++kk) {
-        const int ko = ((kk * 2 + fhalf) ^ ((frow >> 1) & 7)) * 16;
+        const int ko = ((kk * 4 + fq) ^ ((frow >> 1) & 7)) * 16;
         koff_a[kk] = (wm * WROWS + frow) * ROWB + ko;
         koff_w[kk] = (wn * WCOLS + frow) * ROWB + ko;
     }
 
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-    bf16x8 xa[2][MI], wb[2][NJ];
+    bf16x8 xa[2][FM], wb[2][FN];
     // r-th fragment of K-step kk of the slab whose units start at ua / uw, in the order the MFMAs
-    // first need them: x0, w0..w(NJ-1), x1..x(MI-1)
+    // first need them: x0, w0..w(FN-1), x1..x(FM-1)
     auto read_frag = [&](int buf, int ua, int uw, int kk, int r) {
         const char* pa = lds + (ua + koff_a[kk]);
         const char* pw = lds + (uw + koff_w[kk]);
         if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(pa);
-        else if (r <= NJ) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(pw + (r - 1) * 32 * ROWB);
-        else xa[buf][r - NJ] = *reinterpret_cast<const bf16x8*>(pa + (r - NJ) * 32 * ROWB);
+        else if (r <= FN) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(pw + (r - 1) * 16 * ROWB);
+        else xa[buf][r - FN] = *reinterpret_cast<const bf16x8*>(pa + (r - FN) * 16 * ROWB);
     };
     auto mfma_one = [&](int buf, int idx) {
-        const int i = idx / NJ, j = idx % NJ;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
+        const int i = idx / FN, j = idx % FN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
     };
 
     // ua/uw: units of slab kt, ua1/uw1: of slab kt+1, ua2: of A(kt+2); W(kt+2) takes over ua once
@@ -472,17 +469,26 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
                 wait_loads_and_barrier<PU>();  // slab kt+1 is complete in LDS; this slab's units are free
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (stp < 3) {
-                read_frag((stp & 1) ^ 1, ua, uw, stp + 1, r);
-            } else if (r >= BS) {
-                // two per slot: the last one is requested a few MFMAs before the slab ends, so the
-                // wait at the top of the next slab finds it done
-                const int lo = 2 * (r - BS);
-                for (int f = lo; f < lo + 2 && f < READS; ++f) read_frag(0, ua1, uw1, 0, f);
-            }
+            auto slot_reads = [&]() {
+                if (stp < KSUB - 1) {
+                    read_frag((stp & 1) ^ 1, ua, uw, stp + 1, r);
+                } else if (r >= BS) {
+                    // two per slot: the last one is requested a few MFMAs before the slab ends, so the
+                    // wait at the top of the next slab finds it done
+                    const int lo = 2 * (r - BS);
+                    for (int f = lo; f < lo + 2 && f < READS; ++f) read_frag(0, ua1, uw1, 0, f);
+                }
+            };
             // one memory instruction per MFMA interval: the fragment read goes in front of the slot's
-            // first MFMA, the buffer load behind it
+            // first MFMA, the buffer load behind it. The slab's first MFMA waits for the fragments
+            // requested at the end of the previous slab, and that wait is for every outstanding LDS
+            // read: the first read of this slab is therefore issued behind it, not in front.
+            if (s != 0) slot_reads();
             mfma_one(stp & 1, r * PER);
+            if (s == 0) {
+                __builtin_amdgcn_sched_barrier(0);
+                slot_reads();
+            }
             if (s == 1) m3 = slab_mask(kt + 3);
             __builtin_amdgcn_sched_barrier(0);
             if (s % 2 == 0) {
@@ -541,7 +547,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     const int m0 = tm * BM, n0 = tn * BM;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    f32x16 acc[MI][MI];
+    f32x4 acc[2 * MI][2 * MI];
     gemm_tile_slabs<MI>(p, lds, m0, n0, 0, (p.K + BK - 1) / BK, acc);
     gemm_epilogue<MI, MI>(p, acc, lds, m0, n0, wave, lane);
 }
