@@ -363,7 +363,7 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 // Multiplies K slabs [kb, ke) of the tile at (m0, n0) into acc (cleared first). On return every
 // buffer load of the wave has landed and all waves have passed a barrier, so the ring may be
 // reused (the epilogue parks its bf16 blocks there).
-template <int MI>
+template <int MI, bool KTAIL>
 __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, int m0, int n0, int kb, int ke,
                                                 f32x4 (&acc)[2 * MI][2 * MI]) {
     constexpr int NJ = MI;
@@ -392,12 +392,10 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
     const int lrow = tid >> 3;
     const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
     const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BN);
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda), 0,
-        static_cast<int>(((rows_a - 1) * p.lda + p.K) * 2), kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw), 0,
-        static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2), kRsrcFlags);
+    bf16_t* const base_a = const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda);
+    bf16_t* const base_b = const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw);
+    const int bytes_a = static_cast<int>(((rows_a - 1) * p.lda + p.K) * 2);
+    const int bytes_b = static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2);
     uint32_t voff_a[PU], voff_b[PU];
 #pragma unroll
     for (int i = 0; i < PU; ++i) {
@@ -407,15 +405,33 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
     }
     // the slab range ends at ke: everything from there on reads as zeros, like the K tail
     const int k_end = min(p.K, ke * BK);
-    // Slabs past the end and the part of the last slab past K read as zeros: both are "this
-    // thread's chunk starts at or past K" (K is a multiple of 8, so a chunk is all in or all out).
-    auto slab_mask = [&](int kt) -> uint32_t { return kt * BK + lchunk * 8 >= k_end ? kOutOfRange : 0u; };
+    // Slabs past the end and the part of the last slab past K read as zeros. With a K tail (KTAIL)
+    // that is "this thread's chunk starts at or past K" (K is a multiple of 8, so a chunk is all in
+    // or all out) and the mask is a per-lane offset bit. Without one a slab is all in or all out,
+    // the mask is wave-uniform and selects a buffer resource of zero records instead, which keeps
+    // the vector ALU out of the loop.
+    auto slab_mask = [&](int kt) -> uint32_t {
+        if constexpr (KTAIL) return kt * BK + lchunk * 8 >= k_end ? kOutOfRange : 0u;
+        else return kt * BK >= k_end ? kOutOfRange : 0u;
+    };
     // ring offsets are wave-uniform byte offsets of a unit inside the ring
     auto load_a = [&](int uoff, int pass, int kt, uint32_t mask) {
-        load_chunk(rsrc_a, lds + uoff + pass * 4096 + wave * 1024, voff_a[pass] | mask, kt * ROWB);
+        if constexpr (KTAIL) {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_a, 0, bytes_a, kRsrcFlags), lds + uoff + pass * 4096 + wave * 1024,
+                       voff_a[pass] | mask, kt * ROWB);
+        } else {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_a, 0, mask ? 0 : bytes_a, kRsrcFlags),
+                       lds + uoff + pass * 4096 + wave * 1024, voff_a[pass], kt * ROWB);
+        }
     };
     auto load_w = [&](int uoff, int pass, int kt, uint32_t mask) {
-        load_chunk(rsrc_b, lds + uoff + pass * 4096 + wave * 1024, voff_b[pass] | mask, kt * ROWB);
+        if constexpr (KTAIL) {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_b, 0, bytes_b, kRsrcFlags), lds + uoff + pass * 4096 + wave * 1024,
+                       voff_b[pass] | mask, kt * ROWB);
+        } else {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_b, 0, mask ? 0 : bytes_b, kRsrcFlags),
+                       lds + uoff + pass * 4096 + wave * 1024, voff_b[pass], kt * ROWB);
+        }
     };
     // load i of group G(kt) = W(kt+1) then A(kt+2); uw1 / ua2 are the units they go to
     auto group_load = [&](int uw1, int ua2, int i, int kt, uint32_t m1, uint32_t m2) {
@@ -538,7 +554,7 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
 }
 
 
-template <int MI>
+template <int MI, bool KTAIL>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p) {
     constexpr int BM = 64 * MI, BK = 64, NU = 5, UNIT = BM * BK * 2;
     __shared__ __attribute__((aligned(1024))) char lds[NU * UNIT];
@@ -548,7 +564,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     f32x4 acc[2 * MI][2 * MI];
-    gemm_tile_slabs<MI>(p, lds, m0, n0, 0, (p.K + BK - 1) / BK, acc);
+    gemm_tile_slabs<MI, KTAIL>(p, lds, m0, n0, 0, (p.K + BK - 1) / BK, acc);
     gemm_epilogue<MI, MI>(p, acc, lds, m0, n0, wave, lane);
 }
 
@@ -671,7 +687,8 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     p.group_m = 4;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((gemm_nt_ring_kernel<MI>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    if (p.K % 64 == 0) hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, false>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
 // FLUX_GEMM_TILE=256 or 128 forces the tile size (for measurements); anything else = automatic.
