@@ -310,7 +310,7 @@ def main():
         "block_tflops": round(BLOCK_GFLOP / ms_per_step, 1),
         "block_frac_of_mfma_peak": round(BLOCK_GFLOP / ms_per_step / MFMA_PEAK_TFLOPS, 4),
         "roofline": {
-            "kernel": "gemm_nt_ring_kernel<4> (linear1: 4608 x 21504 x 3072, bias, split qkv / GELU(mlp) epilogue)",
+            "kernel": "gemm_nt_ring_kernel<4,false> (linear1: 4608 x 21504 x 3072, bias, split qkv / GELU(mlp) epilogue)",
             "bound": "mfma", "achieved": round(l1_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(l1_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": LINEAR1_TRAFFIC_BYTES,
             "launch_us": round(l1_us, 1), "launches_timed": len(l1_events),
