@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Flux single-stream block on the HIP kernel set (one MI355X).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-kernels] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-kernels] [--no-cpu] [--json-out FILE]
 
 A step is one forward pass of the single-stream block at 4608 tokens (512 txt + 64x64 img),
 hidden 3072, 24 heads, bf16, batch 1, on synthetic seeded inputs that are resident in HBM before
@@ -49,6 +49,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--json-out", default=None, help="also write the result, indented, to this file")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain device-to-device copies of 256 MiB (reference for scaling FETCH_SIZE / "
                          "WRITE_SIZE counter readings), then exit")
@@ -320,9 +321,9 @@ def main():
         result["kernels"] = kernel_table(torch)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
-    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    with open(os.path.join(ROOT, "gpurun_out", "bench_last.json"), "w") as f:
-        json.dump(result, f, indent=1)
+    if args.json_out:
+        with open(args.json_out, "w") as f:
+            json.dump(result, f, indent=1)
     print(json.dumps(result))
 
 
