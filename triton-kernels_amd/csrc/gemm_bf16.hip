@@ -336,17 +336,19 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[
 
 // ------------------------------------------------------------------------------------------------
 // Tiled kernel: 64*MI x 64*MI output tile per workgroup of four waves (2 x 2, a wave owns
-// 32*MI x 32*MI), K in slabs of 64. With two whole-slab LDS stages the memory pipeline would drain
-// at every barrier (the wait in front of it is for ALL outstanding loads) and a slab's last loads
-// would get less than a K=16 step to land. Here LDS is a ring of five units, a unit holding one operand's share of a slab (BM rows x
-// 128 bytes): A(kt) lives in unit 2kt % 5 and W(kt) in unit (2kt+1) % 5. While slab kt is computed,
-// slab kt+1 and A(kt+2) occupy the other three units, so between two barriers the loads of W(kt+1)
-// and A(kt+2) are issued at an even pace, one per four MFMAs, and the wait in front of a barrier
-// only covers W(kt+1): the loads of A(kt+2) stay in flight across it. Every load has between half a
-// slab and a whole slab of MFMA time to land and the memory pipeline never runs empty.
+// 32*MI x 32*MI as (2*MI)^2 accumulators of v_mfma_f32_16x16x32_bf16), K in slabs of 64 = two MFMA
+// steps of K = 32. With two whole-slab LDS stages the memory pipeline would drain at every barrier
+// (the wait in front of it is for ALL outstanding loads). Here LDS is a ring of five units, a unit
+// holding one operand's share of a slab (BM rows x 128 bytes): A(kt) lives in unit 2kt % 5 and
+// W(kt) in unit (2kt+1) % 5. While slab kt is computed, slab kt+1 and A(kt+2) occupy the other
+// three units. The barrier of slab kt sits a quarter into its last step; right behind it the unit
+// of A(kt) is free and takes the loads of W(kt+2), one per slot, and the loads of A(kt+3) follow at
+// an even pace in front of the next barrier. The wait in front of a barrier only covers W of the
+// next slab: the loads of A two slabs ahead stay in flight across it. Every load has more than
+// three quarters of a slab of MFMA time to land and the memory pipeline never runs empty.
 //
-//   slab kt :  step 0   step 1   step 2   step 3 = [MFMA x PER*BS] wait+barrier [rest, reads k0 of kt+1]
-//   loads   :  ......... G(kt) = W(kt+1), A(kt+2) ..........                    | G(kt+1) ...
+//   slab kt :  step 0            step 1 = [MFMA x PER*BS] wait+barrier [rest, reads step 0 of kt+1]
+//   loads   :  ...... A(kt+2) ......................      |  W(kt+2) x PU, one per slot
 //
 // Ring offsets are wave-uniform scalars that advance by two units per slab.
 // ------------------------------------------------------------------------------------------------
@@ -378,8 +380,8 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
     constexpr int BS = READS / 4;                // slots of the last step in front of the barrier
     constexpr int NSLOT = KSUB * READS;          // issue slots per slab
     constexpr int GB = (KSUB - 1) * READS + BS;  // first slot behind the barrier
-    constexpr int EARLY = NL - (GB + 1) / 2;     // loads of a group issued behind the previous slab's barrier
-    static_assert(MFMAS % READS == 0 && KSUB == 2 && NSLOT == 2 * NL && GB % 2 == 0, "schedule shape");
+    constexpr int EARLY = PU;                    // W loads of a group, all issued right behind the previous slab's barrier
+    static_assert(MFMAS % READS == 0 && KSUB == 2 && NSLOT == 2 * NL && NSLOT - GB >= PU, "schedule shape");
     static_assert(2 * (NSLOT - GB) >= READS, "the next slab's first fragments are read two per slot behind the barrier");
     static_assert(4 * WROWS * WCOLS * 2 <= NU * UNIT, "epilogue tile must fit the ring");
     (void)BN; (void)WCOLS;
@@ -433,11 +435,6 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
                        lds + uoff + pass * 4096 + wave * 1024, voff_b[pass], kt * ROWB);
         }
     };
-    // load i of group G(kt) = W(kt+1) then A(kt+2); uw1 / ua2 are the units they go to
-    auto group_load = [&](int uw1, int ua2, int i, int kt, uint32_t m1, uint32_t m2) {
-        if (i < PU) load_w(uw1, i, kt + 1, m1);
-        else load_a(ua2, i - PU, kt + 2, m2);
-    };
 
     // fragment addressing
     // v_mfma_f32_16x16x32_bf16 operand: lane holds row lane % 16, k = (lane / 16) * 8 .. +8 of a K=32 step
@@ -473,9 +470,9 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
     };
 
     // ua/uw: units of slab kt, ua1/uw1: of slab kt+1, ua2: of A(kt+2); W(kt+2) takes over ua once
-    // the barrier has retired it. m1/m2: load masks of slabs kt+1 / kt+2; the mask of slab kt+3 is
+    // the barrier has retired it. m2: load mask of slab kt+2; the mask of slab kt+3 is
     // worked out in the shadow of an MFMA so that the loop back-edge carries register moves only.
-    auto slab = [&](int kt, int ua, int uw, int ua1, int uw1, int ua2, uint32_t m1, uint32_t m2, uint32_t& m3) {
+    auto slab = [&](int kt, int ua, int uw, int ua1, int uw1, int ua2, uint32_t m2, uint32_t& m3) {
         const int uw2 = ua;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -507,9 +504,13 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
             }
             if (s == 1) m3 = slab_mask(kt + 3);
             __builtin_amdgcn_sched_barrier(0);
-            if (s % 2 == 0) {
-                if (s < GB) group_load(uw1, ua2, EARLY + s / 2, kt, m1, m2);
-                else load_w(uw2, (s - GB - GB % 2) / 2, kt + 2, m2);  // first loads of G(kt+1)
+            if (s < GB) {
+                // A(kt+2): PU loads spread evenly over the slots in front of the barrier
+#pragma unroll
+                for (int i = 0; i < PU; ++i)
+                    if ((i * GB) / PU == s) load_a(ua2, i, kt + 2, m2);
+            } else if (s - GB < PU) {
+                load_w(uw2, s - GB, kt + 2, m2);   // W(kt+2): one per slot right behind the barrier
             }
 #pragma unroll
             for (int m = 1; m < PER; ++m) mfma_one(stp & 1, r * PER + m);
@@ -537,14 +538,14 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
 
     {
         int ua = 0, uw = UNIT, ua1 = 2 * UNIT, uw1 = 3 * UNIT, ua2 = 4 * UNIT;
-        uint32_t m1 = slab_mask(kb + 1), m2 = slab_mask(kb + 2);
+        uint32_t m2 = slab_mask(kb + 2);
         for (int kt = kb; kt < ke; ++kt) {
             uint32_t m3;
-            slab(kt, ua, uw, ua1, uw1, ua2, m1, m2, m3);
+            slab(kt, ua, uw, ua1, uw1, ua2, m2, m3);
             // the ring advances by two units
             const int t0 = ua, t1 = uw;
             ua = ua1; uw = uw1; ua1 = ua2; uw1 = t0; ua2 = t1;
-            m1 = m2; m2 = m3;
+            m2 = m3;
         }
     }
     // The last slab's trailing loads were masked (they move no data but still write zeros to LDS):
