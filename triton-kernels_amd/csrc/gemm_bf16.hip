@@ -692,11 +692,12 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
-// FLUX_GEMM_TILE=256 or 128 forces the tile size (for measurements); anything else = automatic.
+// FLUX_GEMM_TILE=256, 128 or 64 forces the tile size (for measurements); anything else = automatic.
 static int forced_tile() {
     static int v = [] {
         const char* e = getenv("FLUX_GEMM_TILE");
-        return e ? atoi(e) : 0;
+        const int t = e ? atoi(e) : 0;
+        return (t == 256 || t == 128 || t == 64) ? t : 0;
     }();
     return v;
 }
@@ -764,8 +765,13 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     // 256 x 256 tiles once they fill most of the 256 CUs; below that 128 x 128 tiles (two workgroups
     // per CU) spread the work better than they lose in operand re-reads.
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+    const int64_t mid_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
     const int tile = forced_tile();
-    if (tile == 256 || (tile != 128 && big_tiles >= 160)) launch_tiled<4>(p, st);
+    // 256-wide tiles once they fill most of the chip; below that 128-wide ones (two workgroups per
+    // CU); problems with too few of those to give every second CU one are bound by the latency of
+    // the K loop and run on 64-wide tiles, four times as many workgroups.
+    if (tile == 256 || (tile == 0 && big_tiles >= 160)) launch_tiled<4>(p, st);
+    else if (tile == 64 || (tile == 0 && mid_tiles <= 64)) launch_tiled<1>(p, st);
     else launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
 }
