@@ -1,8 +1,10 @@
 // Linear layer on the matrix cores:  Y = epilogue(A[M,K] * W[N,K]^T), bf16 operands, fp32 accumulate.
 //
-// Both operands are K-contiguous, which is exactly what v_mfma_f32_32x32x16_bf16 wants: every lane
+// Both operands are K-contiguous, which is exactly what v_mfma_f32_16x16x32_bf16 wants: every lane
 // feeds 8 consecutive k of one row. A workgroup of four waves (2 x 2) owns a (64*MI) x (64*MI) tile
-// of Y and each wave a (32*MI) x (32*MI) sub-tile kept as MI*MI accumulators of 32x32. The K loop
+// of Y and each wave a (32*MI) x (32*MI) sub-tile kept as (2*MI)^2 accumulators of 16x16. (The
+// 16x16x32 shape moves half the accumulator registers per flop of 32x32x16; on a chip that runs
+// this kernel at its power limit that is worth more than the extra instruction issues.) The K loop
 // moves 64-wide slabs of A and W through a five-unit LDS ring (see the kernel) straight from buffer
 // loads that write LDS (no register staging).
 //
