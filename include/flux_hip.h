@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FLUX_ABI_VERSION 1
+#define FLUX_ABI_VERSION 2
 
 enum flux_dtype { FLUX_BF16 = 0, FLUX_F32 = 1 };
 
@@ -135,6 +135,27 @@ int flux_qkv_prep(const flux_qkv_prep_args* args, void* stream);
  * Output columns [0, split_n) go to Y (row stride ldy); columns [split_n, N) go to Y2 at column
  * (n - split_n + y2_col0) with row stride ldy2. split_n == N (or Y2 == null) means one output.
  * ------------------------------------------------------------------------------------------- */
+/* Optional: QK RMSNorm + RoPE applied to the leading columns of a qkv projection on their way out.
+ * Replaces, for q and k, the chain of modules/blocks.py:115-119: the "B L (K H D) -> K B H L D"
+ * rearrange, QKNorm (modules/normalization.py:17-26 over kernels/normalization.py:142-169) and
+ * apply_rope (kernels/positional_embedding.py:55-82).
+ * Output columns [0, heads*128) are the q heads, [heads*128, 2*heads*128) the k heads, 128 columns
+ * each. For those columns y = A W^T + bias is rounded to bf16, normalised over the head
+ * (x * rsqrt(mean x^2 + eps) rounded, times scale rounded), rotated with the 2x2 matrices of its
+ * position (pe[pos][c/2] = [[f00,f01],[f10,f11]] for the column pair c, c+1) and stored at
+ * q_out / k_out [b, head, pos0 + l, :], where row m of the product is (b, l) = (m / seq_len,
+ * m % seq_len). They are not written to Y. Requirements (else FLUX_E_UNSUPPORTED): M and seq_len
+ * multiples of 256, N a multiple of 256, 16-byte aligned pointers, no gate, act_begin and split_n
+ * at or past 2*heads*128, K a multiple of 8. */
+typedef struct flux_linear_qk_fusion {
+    void* q_out; void* k_out;                  /* [B, heads, out_len, 128] bf16, contiguous */
+    const void* q_scale; const void* k_scale;  /* [128] bf16 */
+    const float* pe;                           /* [out_len, 64, 2, 2] fp32 */
+    int64_t pe_batch_stride;                   /* floats between the tables of two batch elements; 0 = one table */
+    int64_t heads, seq_len, out_len, pos0;
+    float eps;
+} flux_linear_qk_fusion;
+
 typedef struct flux_linear_args {
     const void* A; const void* W; const void* bias;
     void* Y; void* Y2;
@@ -144,6 +165,7 @@ typedef struct flux_linear_args {
     int64_t split_n, y2_col0;
     int64_t ldresid, gate_batch_stride, rows_per_batch;
     int32_t act; int64_t act_begin;
+    const flux_linear_qk_fusion* qk;           /* null = off */
 } flux_linear_args;
 
 int flux_linear_bf16(const flux_linear_args* args, void* stream);

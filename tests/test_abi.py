@@ -31,21 +31,23 @@ def test_every_declared_symbol_is_exported_and_bound():
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in flux_hip.h but not exported"
     assert set(names) == set(nv.SIGNATURES), "ctypes binding table and header disagree"
-    assert nv.lib().flux_abi_version() == 1
+    assert nv.lib().flux_abi_version() == 2
 
 
 def test_struct_layouts_match_the_header(tmp_path):
     src = tmp_path / "sizes.c"
     src.write_text(
         '#include <stdio.h>\n#include <stddef.h>\n#include "flux_hip.h"\n'
-        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu %zu\\n\", sizeof(flux_src4), sizeof(flux_qkv_prep_args), "
+        "int main(void){printf(\"%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n\", sizeof(flux_src4), sizeof(flux_qkv_prep_args), "
         "sizeof(flux_linear_args), sizeof(flux_attn_args), offsetof(flux_qkv_prep_args, pe), "
-        "offsetof(flux_linear_args, act_begin), offsetof(flux_attn_args, sm_scale));return 0;}\n")
+        "offsetof(flux_linear_args, act_begin), offsetof(flux_attn_args, sm_scale), sizeof(flux_linear_qk_fusion), "
+        "offsetof(flux_linear_qk_fusion, eps), offsetof(flux_linear_args, qk));return 0;}\n")
     exe = tmp_path / "sizes"
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     got = [int(t) for t in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
     want = [ctypes.sizeof(nv.Src4), ctypes.sizeof(nv.QkvPrepArgs), ctypes.sizeof(nv.LinearArgs), ctypes.sizeof(nv.AttnArgs),
-            nv.QkvPrepArgs.pe.offset, nv.LinearArgs.act_begin.offset, nv.AttnArgs.sm_scale.offset]
+            nv.QkvPrepArgs.pe.offset, nv.LinearArgs.act_begin.offset, nv.AttnArgs.sm_scale.offset,
+            ctypes.sizeof(nv.LinearQKFusion), nv.LinearQKFusion.eps.offset, nv.LinearArgs.qk.offset]
     assert got == want
 
 
@@ -70,7 +72,15 @@ def test_argument_checks_reject_before_launch():
     assert lib.flux_linear_bf16(ctypes.byref(la), None) == -2                                           # lda < K
     la.lda, la.act = 16, 9
     assert lib.flux_linear_bf16(ctypes.byref(la), None) == -6                                           # activation
-    la.act, la.M = 0, 0
+    la.act = 0
+    qf = nv.LinearQKFusion()
+    qf.q_out = qf.k_out = qf.q_scale = qf.k_scale = qf.pe = p
+    qf.heads, qf.seq_len, qf.out_len = 1, 256, 256
+    la.qk = ctypes.pointer(qf)
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == -6                                           # qk fusion on a 4 x 4 product
+    assert b"qk fusion" in lib.flux_last_error()
+    la.qk = None
+    la.M = 0
     assert lib.flux_linear_bf16(ctypes.byref(la), None) == 0                                            # empty
     assert lib.flux_silu(p, p, -1, 0, None) == -2
     qa = nv.QkvPrepArgs()

@@ -38,12 +38,16 @@ def test_single_stream_block(batch_size, seq_len):
     pe = randn(g, 1, 1, seq_len, HEAD_DIM // 2, 2, 2).to(DEV)
     with torch.no_grad():
         y_ref = ref(x=x, vec=vec, pe=pe)
-        y_hip = hip(x=x, vec=vec, pe=pe)
+        y_hip = hip(x=x, vec=vec, pe=pe)              # fused, QKNorm + RoPE in linear1's epilogue
+        hip.fuse_qk_epilogue = False
+        y_prep = hip(x=x, vec=vec, pe=pe)             # fused, QKNorm + RoPE as one kernel behind linear1
         hip.fused = False
         y_unfused = hip(x=x, vec=vec, pe=pe)
     torch.testing.assert_close(y_hip, y_ref, atol=0.1, rtol=0)
+    torch.testing.assert_close(y_prep, y_ref, atol=0.1, rtol=0)
     torch.testing.assert_close(y_unfused, y_ref, atol=0.1, rtol=0)
     torch.testing.assert_close(y_hip, y_unfused, atol=0.05, rtol=0)
+    torch.testing.assert_close(y_hip, y_prep, atol=0.05, rtol=0)
 
 
 @pytest.mark.parametrize("batch_size", [1, 2])

@@ -14,6 +14,7 @@ import torch
 import triton_kernels as tk
 from oracle import flux_oracle as oracle
 from triton_kernels import testing as cfg
+from triton_kernels.kernels import qk_fusable
 from util import DEV, randn, seeded
 
 pytestmark = pytest.mark.gpu
@@ -117,3 +118,46 @@ def test_linear_gated_residual_epilogue(B, L, hid, K):
     y = oracle.linear_ref_fp32(a, w, b).to(torch.bfloat16).view(B, L, hid)
     want = oracle.gated_residual_ref(x, gate, y)
     torch.testing.assert_close(out, want, atol=4e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("B,L,H,mlp,bias,per_batch_pe", [(2, 256, 3, 1152, True, False), (1, 512, 2, 256, False, False),
+                                                         (2, 256, 2, 256, True, True), (1, 4608, 24, 12288, True, False)])
+def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
+    """linear1 with QKNorm + RoPE in the epilogue: q and k leave as [B,H,L,128], v and the GELU'd mlp
+    columns as in the split epilogue. Checked against the oracle chain on the un-fused projection
+    and against the preparation kernel the block otherwise runs."""
+    D, hid = 128, H * 128
+    M, N = B * L, 3 * hid + mlp
+    g = seeded(L + H)
+    x = randn(g, M, hid, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, N, hid, dtype=torch.bfloat16, std=hid ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16, std=0.02).to(DEV) if bias else None
+    qs = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16).to(DEV)
+    ks = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16).to(DEV)
+    pe = randn(g, B if per_batch_pe else 1, 1, L, D // 2, 2, 2).to(DEV)
+
+    qkv = torch.zeros(M, 3 * hid, dtype=torch.bfloat16, device=DEV)
+    both = torch.zeros(M, hid + mlp, dtype=torch.bfloat16, device=DEV)
+    q = torch.empty(B, H, L, D, dtype=torch.bfloat16, device=DEV)
+    k = torch.empty_like(q)
+    assert qk_fusable(x, w, L, D)
+    tk.linear_into(x, w, b, activation="GELU", act_begin=3 * hid, out=qkv, out2=both[:, hid:], split=3 * hid,
+                   qk=dict(q_out=q, k_out=k, q_scale=qs, k_scale=ks, pe=pe, heads=H, seq_len=L, eps=1e-6))
+
+    # un-fused: the same projection, then the preparation kernel
+    qkv_u = torch.empty_like(qkv)
+    both_u = torch.zeros_like(both)
+    tk.linear_into(x, w, b, activation="GELU", act_begin=3 * hid, out=qkv_u, out2=both_u[:, hid:], split=3 * hid)
+    assert torch.equal(qkv[:, 2 * hid:], qkv_u[:, 2 * hid:])           # v columns: same code path, same bits
+    assert torch.equal(both, both_u)
+    assert (qkv[:, :2 * hid] == 0).all()                               # q and k columns are not written
+    heads = qkv_u.view(B, L, 3, H, D).permute(2, 0, 3, 1, 4)
+    q_u, k_u, _ = tk.qkv_prep(heads[0], heads[1], None, pe=pe, q_scale_img=qs, k_scale_img=ks)
+    torch.testing.assert_close(q, q_u, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(k, k_u, atol=1e-2, rtol=1e-2)
+    # oracle chain on the bf16 projection
+    qn = oracle.rms_norm_ref(heads[0].cpu(), qs.cpu())
+    kn = oracle.rms_norm_ref(heads[1].cpu(), ks.cpu())
+    rq, rk = oracle.apply_rope_ref(qn, kn, pe.cpu())
+    torch.testing.assert_close(q.cpu(), rq, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(k.cpu(), rk, atol=2e-2, rtol=2e-2)

@@ -40,6 +40,13 @@ struct GemmParams {
     int tiles_m, tiles_n, group_m;
     int bias_vec;  // 1: bias may be read with 8-byte buffer loads (4-byte aligned base)
     int vec_io;  // 1: every output/residual row segment of 8 columns may be accessed as 16 bytes
+    // fused QK RMSNorm + RoPE for columns [0, qk_cols): q heads first, then k heads, 128 columns each
+    bf16_t* q_out; bf16_t* k_out;
+    const bf16_t* q_scale; const bf16_t* k_scale;
+    const float* pe;
+    int64_t pe_batch_stride;
+    int qk_cols, qk_heads, qk_seq_len, qk_out_len, qk_pos0;
+    float qk_eps;
 };
 
 constexpr int kGemmThreads = 256;
@@ -313,6 +320,135 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x4 (&
     }
 }
 
+// Epilogue for a wave whose 128 columns are one head of q or k: y = A W^T + bias is rounded to bf16
+// (the projection's output), RMS-normalised over the head (x * rstd rounded, times scale rounded),
+// rotated by the 2x2 matrices of its position and written to [B, heads, out_len, 128]. A lane holds
+// 32 of a row's 128 columns; the other 96 are in the lanes 16, 32 and 48 further on, so the sum of
+// squares takes two cross-lane steps. Interior tiles only; a tile lies inside one batch element.
+template <int MI, int NJ>
+__device__ __forceinline__ void gemm_epilogue_qk(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
+                                                 int wave, int lane) {
+    constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
+    static_assert(WCOLS == 128, "a wave's columns are one head of 128");
+    constexpr int C_PITCH = WCOLS * 2, C_CH = WCOLS / 8;
+    constexpr int RPI = 64 / C_CH;
+    constexpr int NIT = 32 / RPI;
+    constexpr int NQ = 2 * NJ;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 15, fq = lane >> 4;
+    char* cw = lds + wave * (WROWS * C_PITCH);
+    const int wave_n0 = n0 + wn * WCOLS;
+    const int wave_m0 = m0 + wm * WROWS;
+    const int hcol = wave_n0 / WCOLS;
+    const bool is_k = hcol >= p.qk_heads;
+    const int head = is_k ? hcol - p.qk_heads : hcol;
+    const int batch = m0 / p.qk_seq_len;                        // the whole tile is in one batch element
+    const int pos_w = p.qk_pos0 + (wave_m0 - batch * p.qk_seq_len);   // output row of the wave's first row
+
+    // bias and scale of this lane's columns stay packed (two bf16 per register) and are unpacked at
+    // their use: the epilogue needs its registers for the rotation entries in flight
+    u32x2 bvp[NQ], scp[NQ];
+    {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(is_k ? p.k_scale : p.q_scale), 0, WCOLS * 2, kRsrcFlags);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) scp[q] = __builtin_amdgcn_raw_buffer_load_b64(rs, (q * 16 + fq * 4) * 2, 0, 0);
+    }
+    if (p.bias != nullptr) {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) bvp[q] = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + q * 16 + fq * 4) * 2, 0, 0);
+    } else {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) bvp[q] = u32x2{0u, 0u};
+    }
+    auto unpack = [](u32x2 v, int e) -> float {
+        const uint32_t w = e < 2 ? v.x : v.y;
+        return __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+    };
+
+    int waddr[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) waddr[q] = frow * C_PITCH + (((q * 2 + (fq >> 1)) ^ (frow & (C_CH - 1))) * 16) + (fq & 1) * 8;
+    const int rrow = lane / C_CH, rch = lane % C_CH;
+    constexpr int NSW = (16 / RPI) < NIT ? (16 / RPI) : NIT;
+    int raddr[NSW];
+#pragma unroll
+    for (int t = 0; t < NSW; ++t) {
+        const int row = t * RPI + rrow;
+        raddr[t] = row * C_PITCH + ((rch ^ (row & (C_CH - 1))) * 16);
+    }
+    // rotation table of this lane's columns: 8 floats per quad, row stride 2 * 128 floats
+    const float* pe_lane = p.pe + static_cast<int64_t>(batch) * p.pe_batch_stride + static_cast<int64_t>(pos_w + frow) * (2 * WCOLS) + fq * 8;
+    char* dst_u = reinterpret_cast<char*>((is_k ? p.k_out : p.q_out) +
+                                          ((static_cast<int64_t>(batch) * p.qk_heads + head) * p.qk_out_len + pos_w) * WCOLS);
+    const uint32_t dst_lane = static_cast<uint32_t>(rrow * (WCOLS * 2) + rch * 16);
+    const float inv_d = 1.0f / static_cast<float>(WCOLS);
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            // the step's rotation entries (from L2) are requested first and land while the sum of
+            // squares is formed; the scheduling barrier keeps the compiler from sinking the loads
+            // to their uses, where each would be waited for in turn
+            f32x4 fr[NQ][2];
+            {
+                const float* pr = pe_lane + (i * 32 + t * 16) * (2 * WCOLS);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    fr[q][0] = *reinterpret_cast<const f32x4*>(pr + q * 32);
+                    fr[q][1] = *reinterpret_cast<const f32x4*>(pr + q * 32 + 4);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // roundings to bf16 two values at a time: one v_cvt_pk_bf16_f32, then the halves widened again
+            auto round2 = [](float a, float b, float& ra, float& rb) {
+                const uint32_t w = pack2_bf16(a, b);
+                ra = __uint_as_float(w << 16);
+                rb = __uint_as_float(w & 0xffff0000u);
+            };
+            float x[NQ][4];
+            float ss = 0.0f;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+                for (int e = 0; e < 4; e += 2)
+                    round2(acc[2 * i + t][q][e] + unpack(bvp[q], e), acc[2 * i + t][q][e + 1] + unpack(bvp[q], e + 1), x[q][e], x[q][e + 1]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ss += x[q][e] * x[q][e];
+            }
+            ss += __shfl_xor(ss, 16);
+            ss += __shfl_xor(ss, 32);
+            const float rstd = rsqrtf(ss * inv_d + p.qk_eps);
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const f32x4 f0 = fr[q][0];
+                const f32x4 f1 = fr[q][1];
+                float xn[4];
+#pragma unroll
+                for (int e = 0; e < 4; e += 2) {
+                    float a, b;
+                    round2(x[q][e] * rstd, x[q][e + 1] * rstd, a, b);
+                    round2(a * unpack(scp[q], e), b * unpack(scp[q], e + 1), xn[e], xn[e + 1]);
+                }
+                const float o0 = f0[0] * xn[0] + f0[1] * xn[1];
+                const float o1 = f0[2] * xn[0] + f0[3] * xn[1];
+                const float o2 = f1[0] * xn[2] + f1[1] * xn[3];
+                const float o3 = f1[2] * xn[2] + f1[3] * xn[3];
+                *reinterpret_cast<u32x2*>(cw + (i * 32 + t * 16) * C_PITCH + waddr[q]) = pack4_bf16(o0, o1, o2, o3);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int row_u = i * 32 + it * RPI;
+            const Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + (i * 32 + (it / NSW) * NSW * RPI) * C_PITCH + raddr[it % NSW]);
+            *reinterpret_cast<Vec16<bf16_t>*>(dst_u + static_cast<int64_t>(row_u) * (WCOLS * 2) + dst_lane) = y;
+        }
+    }
+}
+
 template <int MI, int NJ>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
                                               int wave, int lane) {
@@ -320,6 +456,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[
     const int wave_n0 = n0 + (wave & 1) * WCOLS;
     const bool gelu_all = p.act == FLUX_ACT_GELU_TANH && wave_n0 >= p.act_begin;
     const bool gelu_none = p.act != FLUX_ACT_GELU_TANH || wave_n0 + WCOLS <= p.act_begin;
+    if constexpr (NJ == 4) {
+        if (wave_n0 < p.qk_cols) {   // the host admits the fusion only when every such tile is interior
+            gemm_epilogue_qk<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+            return;
+        }
+    }
     const bool fast = p.vec_io && m0 + BM <= p.M && n0 + BN <= p.N && (gelu_all || gelu_none) &&
                       (wave_n0 + WCOLS <= p.split_n || wave_n0 >= p.split_n) && (p.bias == nullptr || p.bias_vec) &&
                       static_cast<int64_t>(BM) * p.ldy * 2 < 0x7fffffffLL && static_cast<int64_t>(BM) * p.ldy2 * 2 < 0x7fffffffLL;
@@ -738,7 +880,33 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
                (!split || (aligned16(a->Y2) && a->ldy2 % 8 == 0 && a->split_n % 8 == 0 && a->y2_col0 % 8 == 0)) &&
                (!a->gate || (aligned16(a->gate) && aligned16(a->resid) && a->ldresid % 8 == 0 && a->gate_batch_stride % 8 == 0));
 
+    p.q_out = p.k_out = nullptr; p.q_scale = p.k_scale = nullptr; p.pe = nullptr; p.pe_batch_stride = 0;
+    p.qk_cols = p.qk_heads = p.qk_seq_len = p.qk_out_len = p.qk_pos0 = 0; p.qk_eps = 0.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (a->qk != nullptr) {
+        const flux_linear_qk_fusion* f = a->qk;
+        if (!f->q_out || !f->k_out || !f->q_scale || !f->k_scale || !f->pe) return fail(FLUX_E_NULL, "flux_linear_bf16: qk fusion with a null pointer");
+        const int64_t cols = 2 * f->heads * 128;
+        const bool shape_ok = f->heads > 0 && f->seq_len > 0 && f->seq_len % 256 == 0 && a->M % f->seq_len == 0 && a->N % 256 == 0 &&
+                              cols <= a->N && f->pos0 >= 0 && f->pos0 + f->seq_len <= f->out_len && f->out_len < 0x7fffff &&
+                              f->pe_batch_stride >= 0 && a->K > 0 && a->K % 8 == 0;
+        const bool epi_ok = a->gate == nullptr && p.act_begin >= cols && p.split_n >= cols &&
+                            (a->bias == nullptr || p.bias_vec) && p.vec_io;
+        const bool ptr_ok = aligned16(f->q_out) && aligned16(f->k_out) && aligned16(f->pe) && f->pe_batch_stride % 4 == 0 &&
+                            (reinterpret_cast<uintptr_t>(f->q_scale) & 3u) == 0 && (reinterpret_cast<uintptr_t>(f->k_scale) & 3u) == 0 &&
+                            aligned16(a->A) && aligned16(a->W) && a->lda % 8 == 0 && a->ldw % 8 == 0 &&
+                            a->lda * 2 * 256 < 0x7fffffffLL && a->ldw * 2 * 256 < 0x7fffffffLL;
+        if (!shape_ok || !epi_ok || !ptr_ok)
+            return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: qk fusion needs M, N and seq_len in multiples of 256, aligned operands, "
+                                            "no gate, and GELU / split columns behind the k heads");
+        p.q_out = static_cast<bf16_t*>(f->q_out); p.k_out = static_cast<bf16_t*>(f->k_out);
+        p.q_scale = static_cast<const bf16_t*>(f->q_scale); p.k_scale = static_cast<const bf16_t*>(f->k_scale);
+        p.pe = f->pe; p.pe_batch_stride = f->pe_batch_stride;
+        p.qk_cols = (int)cols; p.qk_heads = (int)f->heads; p.qk_seq_len = (int)f->seq_len; p.qk_out_len = (int)f->out_len;
+        p.qk_pos0 = (int)f->pos0; p.qk_eps = f->eps;
+        launch_tiled<4>(p, st);   // a wave's 128 columns are one head
+        return check_launch("flux_linear_bf16");
+    }
     if (p.K == 0) {
         // Degenerate contraction: the scalar kernel's empty K loop leaves bias/epilogue only.
         hipLaunchKernelGGL(gemm_nt_scalar_kernel, dim3((unsigned)(((int64_t)p.M * p.N + 255) / 256)), dim3(256), 0, st, p);

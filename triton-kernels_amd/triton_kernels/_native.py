@@ -40,6 +40,16 @@ class QkvPrepArgs(Structure):
     ]
 
 
+class LinearQKFusion(Structure):
+    _fields_ = [
+        ("q_out", c_void_p), ("k_out", c_void_p),
+        ("q_scale", c_void_p), ("k_scale", c_void_p),
+        ("pe", c_void_p), ("pe_batch_stride", c_int64),
+        ("heads", c_int64), ("seq_len", c_int64), ("out_len", c_int64), ("pos0", c_int64),
+        ("eps", c_float),
+    ]
+
+
 class LinearArgs(Structure):
     _fields_ = [
         ("A", c_void_p), ("W", c_void_p), ("bias", c_void_p),
@@ -50,6 +60,7 @@ class LinearArgs(Structure):
         ("split_n", c_int64), ("y2_col0", c_int64),
         ("ldresid", c_int64), ("gate_batch_stride", c_int64), ("rows_per_batch", c_int64),
         ("act", c_int32), ("act_begin", c_int64),
+        ("qk", POINTER(LinearQKFusion)),
     ]
 
 
@@ -105,7 +116,7 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.flux_abi_version() != 1:
+        if handle.flux_abi_version() != 2:
             raise RuntimeError("libfluxhip.so: ABI version mismatch")
         _lib = handle
     return _lib

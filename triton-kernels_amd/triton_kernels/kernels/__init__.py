@@ -1,7 +1,7 @@
 """Operator entry points: thin Python launchers over the C ABI of libfluxhip.so."""
 from triton_kernels.kernels.normalization import layer_norm_modulation, rms_norm
 from triton_kernels.kernels.positional_embedding import apply_rope, qkv_prep
-from triton_kernels.kernels.linear import linear, linear_into
+from triton_kernels.kernels.linear import linear, linear_into, qk_fusable
 from triton_kernels.kernels.attention import attention_into, scaled_dot_product_attention
 
 __all__ = [

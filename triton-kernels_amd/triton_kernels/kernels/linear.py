@@ -2,6 +2,8 @@
 with the extra epilogues the fused Flux blocks use."""
 from __future__ import annotations
 
+import ctypes
+
 import torch
 from torch import Tensor
 
@@ -9,7 +11,7 @@ from triton_kernels import _native as nv
 
 _ACTIVATIONS = {"": nv.ACT_NONE, "GELU": nv.ACT_GELU_TANH}
 # Tile plan per dtype; like the reference's table it has a single entry, so any other dtype is a KeyError.
-_PLANS = {torch.bfloat16: {"tile": (256, 256, 64), "waves": 4, "mfma": "32x32x16"}}
+_PLANS = {torch.bfloat16: {"tile": (256, 256, 64), "waves": 4, "mfma": "16x16x32"}}
 
 
 def _rows_2d(x: Tensor, K: int) -> Tensor:
@@ -23,13 +25,17 @@ def _rows_2d(x: Tensor, K: int) -> Tensor:
 
 def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "", act_begin: int = 0,
                 out: Tensor | None = None, out2: Tensor | None = None, split: int | None = None,
-                resid: Tensor | None = None, gate: Tensor | None = None) -> Tensor:
+                resid: Tensor | None = None, gate: Tensor | None = None, qk: dict | None = None) -> Tensor:
     """General form of the fused linear.
 
     out   : [M, >=split] destination (row stride free) for columns [0, split)
     out2  : destination for columns [split, N), written starting at its column 0
     act_begin : GELU applies to columns >= act_begin only
     resid, gate : y = resid + gate * y with resid [..., N] and gate [B, 1, N] (or [B, N])
+    qk    : QK RMSNorm + RoPE on the way out for the leading 2 * heads * 128 columns (q heads, then k
+            heads), which then go to q_out / k_out [B, heads, out_len, 128] instead of `out`:
+            dict(q_out, k_out, q_scale, k_scale, pe, heads, seq_len, pos0=0, eps=1e-6); see
+            qk_fusable() for the shapes this form takes
     """
     assert x.shape[-1] == w.shape[-1], "Incompatible dimensions"
     assert x.dtype == w.dtype, "Incompatible dtypes"
@@ -74,10 +80,37 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
         a.resid, a.ldresid = r2.data_ptr(), r2.stride(0)
         a.gate, a.gate_batch_stride, a.rows_per_batch = g2.data_ptr(), (g2.stride(0) if nb > 1 else N), M // nb
     a.act, a.act_begin = act, act_begin
+    keep = None
+    if qk is not None:
+        f = nv.LinearQKFusion()
+        q_out, k_out, pe = qk["q_out"], qk["k_out"], qk["pe"]
+        heads, seq_len = int(qk["heads"]), int(qk["seq_len"])
+        assert q_out.is_contiguous() and k_out.is_contiguous() and q_out.shape == k_out.shape and q_out.dtype == x.dtype
+        assert q_out.dim() == 4 and q_out.shape[1] == heads and q_out.shape[3] == 128 and M % seq_len == 0 and q_out.shape[0] == M // seq_len
+        out_len = q_out.shape[2]
+        pe2 = pe.reshape(-1, out_len, 64, 2, 2)
+        assert pe2.dtype == torch.float32 and pe2.is_contiguous()
+        qs, ks = qk["q_scale"].to(x.dtype).contiguous(), qk["k_scale"].to(x.dtype).contiguous()
+        f.q_out, f.k_out, f.q_scale, f.k_scale = q_out.data_ptr(), k_out.data_ptr(), qs.data_ptr(), ks.data_ptr()
+        f.pe, f.pe_batch_stride = pe2.data_ptr(), (pe2.stride(0) if pe2.shape[0] > 1 else 0)
+        f.heads, f.seq_len, f.out_len, f.pos0 = heads, seq_len, out_len, int(qk.get("pos0", 0))
+        f.eps = float(qk.get("eps", 1e-6))
+        a.qk = ctypes.pointer(f)
+        keep = (f, qs, ks, pe2)
     with nv.on_device(dev):
         rc = nv.lib().flux_linear_bf16(nv.byref(a), nv.stream_ptr(dev))
     nv.check(rc, "flux_linear_bf16")
+    del keep
     return out
+
+
+def qk_fusable(x: Tensor, w: Tensor, seq_len: int, head_dim: int) -> bool:
+    """Whether linear_into(..., qk=...) takes this projection: bf16, heads of 128, and rows, columns
+    and sequence length in multiples of the 256-wide tile (so every q/k tile is interior and lies
+    inside one batch element)."""
+    M = x.numel() // x.shape[-1]
+    return (x.dtype == torch.bfloat16 and head_dim == 128 and seq_len > 0 and seq_len % 256 == 0 and M % seq_len == 0
+            and w.shape[0] % 256 == 0 and w.shape[1] % 8 == 0)
 
 
 def linear(x: Tensor, w: Tensor, b: Tensor | None, activation: str = "") -> Tensor:

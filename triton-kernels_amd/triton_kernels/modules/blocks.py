@@ -25,7 +25,7 @@ from torch import Tensor
 
 from triton_kernels import _native as nv
 from triton_kernels.kernels.attention import attention_into, scaled_dot_product_attention
-from triton_kernels.kernels.linear import linear, linear_into
+from triton_kernels.kernels.linear import linear, linear_into, qk_fusable
 from triton_kernels.kernels.normalization import layer_norm_modulation
 from triton_kernels.kernels.positional_embedding import apply_rope, qkv_prep
 from triton_kernels.modules.normalization import QKNorm
@@ -152,6 +152,9 @@ class SingleStreamBlock(nn.Module):
     """DiT block with parallel attention and MLP branches (https://arxiv.org/abs/2302.05442)."""
 
     fused = True
+    # QKNorm + RoPE inside linear1's epilogue when the shapes allow (heads of 128, sequence length a
+    # multiple of 256); otherwise, or with this switched off, one preparation kernel behind linear1
+    fuse_qk_epilogue = True
 
     def __init__(self, hidden_size: int, num_heads: int, mlp_ratio: float = 4.0, qk_scale: float | None = None):
         super().__init__()
@@ -187,12 +190,24 @@ class SingleStreamBlock(nn.Module):
         qkv = torch.empty((B, L, 3 * hid), dtype=x.dtype, device=x.device)
         both = torch.empty((B, L, hid + self.mlp_hidden_dim), dtype=x.dtype, device=x.device)
         both2 = both.view(M, -1)
-        # linear1: qkv columns -> qkv, mlp columns -> GELU -> both[:, hid:]
-        linear_into(x_mod, self.linear1.weight, self.linear1.bias, activation="GELU", act_begin=3 * hid,
-                    out=qkv.view(M, -1), out2=both2[:, hid:], split=3 * hid)
-        q_src, k_src, v_src = _heads(qkv, H)
-        q, k, _ = qkv_prep(q_src, k_src, None, pe=pe,
-                           q_scale_img=self.norm.query_norm.scale, k_scale_img=self.norm.key_norm.scale)
+        _, _, v_src = _heads(qkv, H)
+        pe_ok = pe.dtype == torch.float32 and pe.is_contiguous() and pe.numel() in (L * D * 2, B * L * D * 2)
+        if self.fuse_qk_epilogue and pe_ok and qk_fusable(x_mod, self.linear1.weight, L, D):
+            # linear1: q and k columns -> bias, RMSNorm, RoPE -> q, k [B,H,L,D]; v columns -> qkv;
+            # mlp columns -> GELU -> both[:, hid:]
+            q = torch.empty((B, H, L, D), dtype=x.dtype, device=x.device)
+            k = torch.empty_like(q)
+            linear_into(x_mod, self.linear1.weight, self.linear1.bias, activation="GELU", act_begin=3 * hid,
+                        out=qkv.view(M, -1), out2=both2[:, hid:], split=3 * hid,
+                        qk=dict(q_out=q, k_out=k, q_scale=self.norm.query_norm.scale, k_scale=self.norm.key_norm.scale,
+                                pe=pe, heads=H, seq_len=L, eps=1e-6))
+        else:
+            # linear1: qkv columns -> qkv, mlp columns -> GELU -> both[:, hid:]
+            linear_into(x_mod, self.linear1.weight, self.linear1.bias, activation="GELU", act_begin=3 * hid,
+                        out=qkv.view(M, -1), out2=both2[:, hid:], split=3 * hid)
+            q_src, k_src, _ = _heads(qkv, H)
+            q, k, _ = qkv_prep(q_src, k_src, None, pe=pe,
+                               q_scale_img=self.norm.query_norm.scale, k_scale_img=self.norm.key_norm.scale)
         # attention output lands in both[:, :hid] in "B L (H D)" order
         attn_out = both[..., :hid].view(B, L, H, D).permute(0, 2, 1, 3)
         attention_into(q, k, v_src, attn_out)
