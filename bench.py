@@ -37,9 +37,9 @@ LINEAR1_FLOP = 2.0 * 4608 * 21504 * 3072
 
 # Fabric-side traffic of one linear1 launch (what the L2s fetch from / write to Infinity Cache + HBM),
 # from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script, each scaled by what
-# the same counter reads for a plain 256 MiB copy (`--calibrate-copy`): fetch 509655.0 x 2.000 KiB,
+# the same counter reads for a plain 256 MiB copy (`--calibrate-copy`): fetch 557483.0 x 2.000 KiB,
 # write 193536.0 x 1.000 KiB per dispatch. The summary is profiles/gemm_linear1_linear2_4608_hbm_traffic.md.
-LINEAR1_TRAFFIC_BYTES = int((509655.0 * 2.000 + 193536.0 * 1.000) * 1024)
+LINEAR1_TRAFFIC_BYTES = int((557483.0 * 2.000 + 193536.0 * 1.000) * 1024)
 
 
 def parse_args():
