@@ -140,7 +140,7 @@ def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
     both = torch.zeros(M, hid + mlp, dtype=torch.bfloat16, device=DEV)
     q = torch.empty(B, H, L, D, dtype=torch.bfloat16, device=DEV)
     k = torch.empty_like(q)
-    assert qk_fusable(x, w, L, D)
+    assert qk_fusable(x, w, L, D) == ((M // 256) * (N // 256) >= 160)   # small ones are taken, just not preferred
     tk.linear_into(x, w, b, activation="GELU", act_begin=3 * hid, out=qkv, out2=both[:, hid:], split=3 * hid,
                    qk=dict(q_out=q, k_out=k, q_scale=qs, k_scale=ks, pe=pe, heads=H, seq_len=L, eps=1e-6))
 
