@@ -76,7 +76,7 @@ __device__ __forceinline__ void lds_load16_raw(u32x4 rsrc, uint32_t lds_addr, ui
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
-                 : "memory");  // m0 is written; nothing else in this file's kernel reads it (LDS ops need no m0 on gfx9+)
+                 : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p));
@@ -168,6 +168,11 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
         for (int kk = 0; kk < KSTEPS; ++kk) {
             u32x4 t = *reinterpret_cast<const u32x4*>(rp + (kk * 2 + fhalf) * 8);
             if (!ok) t = u32x4{0u, 0u, 0u, 0u};
+            // sm_scale*log2(e) goes into Q once (rounded to bf16), so scores leave the MFMA in the
+            // base-2 domain whatever the sign of the scale, and masked keys stay -inf for scale 0
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                t[e] = pack2_bf16(__uint_as_float(t[e] << 16) * p.scale_log2, __uint_as_float(t[e] & 0xffff0000u) * p.scale_log2);
             qf[qb][kk] = __builtin_bit_cast(bf16x8, t);
         }
     }
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[qb][db][r] = 0.0f;
     }
-    const float c = p.scale_log2;
+    constexpr float c = 1.0f;  // the scale is already in Q
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int ntiles = (p.L + BN - 1) / BN;
 
@@ -438,12 +443,548 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Head dim 128, 64 query rows per wave, one wave per SIMD, v_mfma_f32_16x16x32_bf16.
+//
+// The kernel above gives every wave 32 query rows, so a wave reads a whole K and a whole V tile
+// from LDS for 32 rows' worth of MFMA work; at full MFMA rate that is more than the LDS can
+// deliver (the transposing V^T reads run at about 70 bytes per clock per CU). Here a wave owns 64
+// rows (four 16-row blocks), every K / V^T fragment feeds four MFMAs, and LDS traffic per flop
+// halves. The price is the register file: 128 accumulator registers for O^T, 64 for Q, two S^T
+// buffers and two P^T buffers need more than 256, so one wave per SIMD runs and the instruction
+// stream itself has to keep the matrix pipe fed, the way a GEMM main loop does.
+//
+//   * Work is cut into sub-tiles of 32 keys. Iteration u issues 64 MFMAs: 32 for S^T(u+1) =
+//     K(u+1) Q^T and 32 for O^T += V(u-1)^T P(u-1)^T, while the VALU turns S^T(u) into P^T(u), one
+//     VALU instruction behind each MFMA. LDS fragment reads are issued eight slots ahead of use.
+//   * Q is scaled by sm_scale*log2(e) and rounded to bf16 once; the first MFMA of every S^T
+//     accumulator takes "-m" (the row's reference maximum, one register block per 16 rows) as its
+//     C operand, so exp2 applies to the MFMA result directly: no multiply, no subtract.
+//   * The reference maximum is not the running maximum: it is only moved when a row's partial sum
+//     of a sub-tile exceeds 2^40 (which also catches inf). exp2(s - m) is then simply larger than
+//     one for a while, which costs no accuracy in fp32 / bf16 (relative precision), and the common
+//     path has no max, no compare per element and no rescale. When the test fires (first sub-tile
+//     aside this needs scores to grow by more than 40 in the log2 domain) the whole wave
+//     re-bases: true row maxima, accumulators, sums and the S^T blocks in flight are shifted.
+//   * K and V tiles of 64 keys go through two LDS rings of four (128 KB) so that every LDS offset
+//     in the four-tile body is a compile-time constant; one workgroup barrier per 64 keys.
+// ------------------------------------------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// MFMAs of this kernel are issued from inline asm so that the register file is laid out by hand.
+// Left to the compiler, a kernel with more than 256 registers gets accumulation-register MFMAs for
+// everything and a copy in front of every VALU use, or keeps the "a"-constrained operands in vector
+// registers and copies them over in front of every MFMA.
+//   * The accumulation registers are addressed by number: a[0:127] = O^T accumulators, block
+//     (db, qb) at a[16*db + 4*qb ..+3]; a[128:191] = Q fragments, (qb, ks) at a[128 + 16*qb + 4*ks ..+3].
+//     The compiler never sees them (attn_claim_agprs only makes the kernel descriptor reserve
+//     them), so it must not use accumulation registers of its own: the kernel has to fit the 256
+//     vector registers without spilling, which tests/test_abi.py checks on the generated code.
+//   * S^T, P^T and the LDS fragments are ordinary variables in vector registers (the VALU reads and
+//     writes them every slot).
+// The hardware does not interlock an MFMA result against a VALU access that follows too closely,
+// and the compiler takes an asm statement for an instruction that is complete when the next one
+// issues: in the main loop every such pair is half an iteration apart by construction, the rare
+// paths (prologue, re-base, epilogue) wait explicitly, and every vector register an MFMA reads or
+// writes keeps that role for the whole loop (keep_regs in front of each redefinition), so that the
+// compiler cannot hand it to a VALU temporary while an MFMA that uses it is still queued.
+#define ATTN_A16(b) "a" #b "0", "a" #b "1", "a" #b "2", "a" #b "3", "a" #b "4", "a" #b "5", "a" #b "6", "a" #b "7", "a" #b "8", "a" #b "9"
+__device__ __forceinline__ void attn_claim_agprs() {
+    asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", ATTN_A16(1), ATTN_A16(2), ATTN_A16(3),
+                 ATTN_A16(4), ATTN_A16(5), ATTN_A16(6), ATTN_A16(7), ATTN_A16(8), ATTN_A16(9), ATTN_A16(10), ATTN_A16(11),
+                 ATTN_A16(12), ATTN_A16(13), ATTN_A16(14), ATTN_A16(15), ATTN_A16(16), ATTN_A16(17), ATTN_A16(18), "a190", "a191");
+}
+#undef ATTN_A16
+constexpr int kAccQ = 128;  // first accumulation register of the Q fragments
+// S^T block (vector registers) = K fragment x Q fragment (accumulation registers QLO..QLO+3) + c
+template <int QLO>
+__device__ __forceinline__ void mfma_s_seed(f32x4& d, const bf16x8& a, const f32x4& c) {
+    // "+v" on the destination although the old value is not read: the block keeps its registers
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, a[%3:%4], %2" : "+v"(d) : "v"(a), "v"(c), "n"(QLO), "n"(QLO + 3));
+}
+// The same with C = 0 as an inline constant. (A register holding zeros would be written by a VALU
+// move that the compiler may place right in front of the asm: the MFMA would read it too early.)
+template <int QLO>
+__device__ __forceinline__ void mfma_s_zero(f32x4& d, const bf16x8& a) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, a[%2:%3], 0" : "+v"(d) : "v"(a), "n"(QLO), "n"(QLO + 3));
+}
+template <int QLO>
+__device__ __forceinline__ void mfma_s_acc(f32x4& d, const bf16x8& a) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, a[%2:%3], %0" : "+v"(d) : "v"(a), "n"(QLO), "n"(QLO + 3));
+}
+// O^T block (accumulation registers OLO..OLO+3) += V^T fragment x P^T fragment
+template <int OLO>
+__device__ __forceinline__ void mfma_o_acc(const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(a), "v"(b), "n"(OLO), "n"(OLO + 3));
+}
+template <int R> __device__ __forceinline__ void acc_write(uint32_t v) {
+    asm volatile("v_accvgpr_write_b32 a[%1], %0" : : "v"(v), "n"(R));
+}
+template <int R> __device__ __forceinline__ float acc_read() {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(R));
+    return v;
+}
+// Marks the old value of x as used here, so that its registers stay reserved up to this point.
+template <typename T> __device__ __forceinline__ void keep_regs(T& x) { asm volatile("" : "+v"(x)); }
+// Enough wait states for the newest MFMA result to be readable by the VALU (and the other way round).
+__device__ __forceinline__ void mfma_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+// Wait states between VALU writes of the four seed blocks and the MFMAs that read them.
+__device__ __forceinline__ void mfma_settle_seeds(f32x4 (&b)[4]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : : "memory");
+}
+// The same, and the compiler may not move a use of the S^T blocks in b across it (register-only
+// code is otherwise free to float above an asm statement it has no operand in common with).
+template <int QB>
+__device__ __forceinline__ void mfma_settle(f32x4 (&b)[2][QB]) {
+    static_assert(QB == 4, "operand list");
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[1][2]), "+v"(b[1][3])
+                 :
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void attn_vmwait_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// VALU work of one iteration as a list of 81 single-instruction steps, spread over the first 60 of
+// the 64 MFMA slots. A unit is two scores of one query block: E0, E1 = their exponentials, C = pack
+// to bf16, A0, A1 = add to the row sum (fp32, from the unrounded values: the dot-product
+// instructions that would sum the rounded pair share the matrix pipe with the MFMAs and cost a
+// whole MFMA slot each). Steps of unit k-1 are interleaved with the exponentials of unit k so that
+// no step waits for the one before it and two exponentials never fall into one slot.
+enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_CHECK };
+constexpr int kAttnSteps = 81;
+constexpr int attn_step_kind(int j) {
+    if (j < 2) return j == 0 ? ATT_E0 : ATT_E1;
+    if (j >= 77) return j == 77 ? ATT_C : j == 78 ? ATT_A0 : j == 79 ? ATT_A1 : ATT_CHECK;
+    constexpr int order[5] = {ATT_E0, ATT_C, ATT_E1, ATT_A0, ATT_A1};
+    return order[(j - 2) % 5];
+}
+constexpr int attn_step_unit(int j) {
+    if (j < 2) return 0;
+    if (j >= 77) return 15;
+    const int k = 1 + (j - 2) / 5, kind = attn_step_kind(j);
+    return (kind == ATT_E0 || kind == ATT_E1) ? k : k - 1;
+}
+constexpr int attn_step_slot(int j) { return j < 2 ? j : 2 + ((j - 2) * 58) / 79; }
+constexpr int attn_first_step(int slot) {  // steps of a slot are consecutive in the list
+    for (int j = 0; j < kAttnSteps; ++j)
+        if (attn_step_slot(j) == slot) return j;
+    return kAttnSteps;
+}
+constexpr int attn_step_count(int slot) {
+    int n = 0;
+    for (int j = 0; j < kAttnSteps; ++j) n += attn_step_slot(j) == slot;
+    return n;
+}
+
+__global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
+    constexpr int D = 128, QB = 4, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
+    constexpr int V0 = 4 * TB;
+    constexpr float kRebase = 1.0995116e12f;  // 2^40
+    __shared__ __attribute__((aligned(1024))) char lds[8 * TB + 4096];  // K ring of 4 tiles, V ring of 4 tiles, 1 KB per wave for the re-base
+
+    const int per_xcd = gridDim.x / 8;
+    const int vt = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (vt >= p.total_tiles) return;
+    const int bh = vt / p.n_qtiles, qt = vt % p.n_qtiles;
+    const int b = bh / p.H, h = bh % p.H;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int q0 = qt * 256 + wave * 64;
+    const float c = p.scale_log2;
+#ifdef X_CLOCKS
+    const long long x_t0 = clock64(), x_w0 = wall_clock64();
+#endif
+
+    const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
+    const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
+
+    // loader: a wave-wide load is 4 rows x 256 bytes; pass i covers rows i*16 + wave*4 + lane/16.
+    // LDS position pos of row r holds the 16-byte chunk pos ^ (r & 15) of a K row (fragment reads
+    // take one chunk of 16 consecutive rows) and chunk pos ^ ((r & 7) << 1) of a V row (transposing
+    // reads take 32-byte pieces of 4 consecutive rows in each of four lane groups).
+    const int l_row = lane >> 4, l_pos = lane & 15;
+    uint32_t k_voff[4], v_voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i * 16 + wave * 4 + l_row;
+        k_voff[i] = static_cast<uint32_t>((r * p.k_sl + ((l_pos ^ (r & 15)) * 8)) * 2);
+        v_voff[i] = static_cast<uint32_t>((r * p.v_sl + ((l_pos ^ ((r & 7) << 1)) * 8)) * 2);
+    }
+    const int k_row2 = static_cast<int>(p.k_sl * 2), v_row2 = static_cast<int>(p.v_sl * 2);
+    auto tile_rsrc = [&](const bf16_t* base, int row2, int key0) -> u32x4 {
+        const int rows = min(p.L - key0, 64);
+        const int bytes = rows > 0 ? (rows - 1) * row2 + D * 2 : 0;
+        const uint64_t addr = reinterpret_cast<uint64_t>(base) + static_cast<uint64_t>(static_cast<int64_t>(key0) * row2);
+        u32x4 r;
+        r.x = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr));
+        r.y = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr >> 32) & 0xffffu);
+        r.z = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bytes));
+        r.w = kAttnRsrcFlags;
+        return r;
+    };
+    const uint32_t lds_base = lds_addr_of(lds) + wave * 1024;
+    const uint32_t scr_addr = lds_addr_of(lds) + 8 * TB + tid * 16;
+    auto load_k = [&](int tile, int buf) {
+        const u32x4 rs = tile_rsrc(kbase, k_row2, tile * 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds_load16_raw(rs, lds_base + buf * TB + i * 4096, k_voff[i]);
+    };
+    auto load_v = [&](int tile, int buf) {
+        const u32x4 rs = tile_rsrc(vbase, v_row2, tile * 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds_load16_raw(rs, lds_base + V0 + buf * TB + i * 4096, v_voff[i]);
+    };
+
+    // The first pass through the loop multiplies P = 0 with whatever the last V buffer holds:
+    // make that finite.
+    {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds + V0 + 3 * TB + i * 4096 + tid * 16) = z;
+    }
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+
+    // Q fragments ("B" operand of S^T): lane holds row q0 + qb*16 + r16, d = ks*32 + g*8 .. +8,
+    // scaled by sm_scale*log2(e) and rounded to bf16.
+    attn_claim_agprs();
+    {
+        u32x4 qraw[QB][KS];  // all sixteen loads in flight before the first conversion
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            const int row = q0 + qb * 16 + r16;
+            const bool ok = row < p.L;
+            const bf16_t* rp = p.q + b * p.q_sb + h * p.q_sh + static_cast<int64_t>(ok ? row : 0) * p.q_sl;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                qraw[qb][ks] = *reinterpret_cast<const u32x4*>(rp + ks * 32 + g * 8);
+                if (!ok) qraw[qb][ks] = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        static_for<0, QB * KS * 4>([&](auto i_c) {
+            constexpr int i = decltype(i_c)::value, qb = i / 16, ks = (i / 4) % 4, e = i % 4;
+            const uint32_t t = qraw[qb][ks][e];
+            acc_write<kAccQ + i>(pack2_bf16(__uint_as_float(t << 16) * c, __uint_as_float(t & 0xffff0000u) * c));
+        });
+        static_for<0, 128>([&](auto i_c) { acc_write<decltype(i_c)::value>(0u); });  // O^T = 0
+    }
+
+    // fragment addresses, lane part (the ring offset of the sub-tile is added once per iteration,
+    // key-block and second-read offsets are immediates)
+    // K ("A" of S^T): row kb*16 + r16 of the sub-tile, chunk ks*4 + g.
+    // V^T ("A" of O^T): lane group g transposes key rows g*4 .. g*4+3 (first read) and 16 + g*4 ..
+    // (second read) of the sub-tile; lane r16 points at row g*4 + r16/4, 8 bytes at d = db*16 + (r16%4)*4.
+    int k_addr[KS], v_addr[DBN];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = r16 * ROWB + (((ks * 4 + g) ^ r16) * 16);
+    {
+        const int rr = r16 >> 2, cc = r16 & 3, row = g * 4 + rr;
+#pragma unroll
+        for (int db = 0; db < DBN; ++db) v_addr[db] = V0 + row * ROWB + ((db ^ (row & 7)) * 32) + cc * 8;
+    }
+
+    f32x4 seed[QB];   // -m of the row, in every register of the block: C operand of the first S^T MFMA
+    float l_run[QB];
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        seed[qb] = zero4;
+        l_run[qb] = 0.0f;
+    }
+    const int ntiles = (p.L + 63) / 64;
+
+    // Every register an MFMA reads or writes is kept for that purpose through the whole loop
+    // (keep_regs in front of each redefinition): see mfma_s_seed.
+    bf16x8 kf[4];
+    s16x4 vlo[4], vhi[4];
+    f32x4 s0[2][QB], s1[2][QB];
+    uint32_t pw0[QB][4], pw1[QB][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        kf[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        vlo[i] = s16x4{0, 0, 0, 0};
+        vhi[i] = s16x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) pw0[qb][w] = pw1[qb][w] = 0u;
+        s0[0][qb] = s0[1][qb] = s1[0][qb] = s1[1][qb] = zero4;
+    }
+    int ka_a[KS], ka_b[KS], va[DBN];  // K fragment addresses of two consecutive sub-tiles, V^T of one
+    auto read_k = [&](const int (&ka)[KS], int n) {  // n-th K fragment of a sub-tile: key block n/4, d step n%4
+        keep_regs(kf[n % 4]);
+        kf[n % 4] = *reinterpret_cast<const bf16x8*>(lds + ka[n % 4] + (n / 4) * 16 * ROWB);
+    };
+    auto vfrag = [&](int m) {
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 both = {vlo[m][0], vlo[m][1], vlo[m][2], vlo[m][3], vhi[m][0], vhi[m][1], vhi[m][2], vhi[m][3]};
+        return __builtin_bit_cast(bf16x8, both);
+    };
+
+    // ---- prologue: S^T(0) from the first half of K(0), then the rows' first reference maxima
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+        const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % 4] + (n / 4) * 16 * ROWB);
+        static_for<0, QB>([&](auto qb_c) {
+            constexpr int qb = decltype(qb_c)::value;
+            if (n % 4 == 0) mfma_s_zero<kAccQ + 16 * qb>(s0[n / 4][qb], f);
+            else if (n % 4 == 1) mfma_s_acc<kAccQ + 16 * qb + 4>(s0[n / 4][qb], f);
+            else if (n % 4 == 2) mfma_s_acc<kAccQ + 16 * qb + 8>(s0[n / 4][qb], f);
+            else mfma_s_acc<kAccQ + 16 * qb + 12>(s0[n / 4][qb], f);
+        });
+    }
+    mfma_settle(s0);
+    load_k(2, 2);
+    load_v(1, 1);
+    load_k(3, 3);
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int key = kb * 16 + g * 4 + j;
+                if (key >= p.L) s0[kb][qb][j] = -INFINITY;
+                mx = fmaxf(mx, s0[kb][qb][j]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) seed[qb][j] = -mx;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) s0[kb][qb] -= mx;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ka_a[ks] = k_addr[ks] + HALF;  // second half of K(0)
+    mfma_settle_seeds(seed);
+    read_k(ka_a, 0);
+    read_k(ka_a, 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Shift the reference maxima of all rows of the wave (rare). sc = S^T of the sub-tile whose
+    // sums tripped the test, sn = the complete S^T of the next one (seeded with the old reference).
+    auto rebase = [&](f32x4 (&sc)[2][QB], f32x4 (&sn)[2][QB], uint32_t (&pw)[QB][4], float (&sum)[QB]) {
+        mfma_settle(sc);
+        mfma_settle(sn);
+        static_for<0, QB>([&](auto qb_c) {
+            constexpr int qb = decltype(qb_c)::value, QBC = qb;
+            float mx = fmaxf(fmaxf(sc[0][qb][0], sc[0][qb][1]), fmaxf(sc[0][qb][2], sc[0][qb][3]));
+            mx = fmaxf(mx, fmaxf(fmaxf(sc[1][qb][0], sc[1][qb][1]), fmaxf(sc[1][qb][2], sc[1][qb][3])));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float d = fmaxf(mx, 0.0f);  // the reference only ever moves up
+            const float f = __builtin_amdgcn_exp2f(-d);
+            seed[qb] -= d;
+            l_run[qb] *= f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                sc[kb][qb] -= d;
+                sn[kb][qb] -= d;
+            }
+            static_for<0, DBN * 4>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value, r = 16 * (i / 4) + 4 * QBC + i % 4;
+                acc_write<r>(__float_as_uint(acc_read<r>() * f));
+            });
+            float sm = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float p0 = __builtin_amdgcn_exp2f(sc[w / 2][qb][(w % 2) * 2]);
+                const float p1 = __builtin_amdgcn_exp2f(sc[w / 2][qb][(w % 2) * 2 + 1]);
+                pw[qb][w] = pack2_bf16(p0, p1);
+                sm += p0 + p1;
+            }
+            sum[qb] = sm;
+        });
+        mfma_settle_seeds(seed);
+    };
+
+    // One iteration = 64 slots of (MFMA, fragment reads for later slots, VALU steps of the softmax).
+    //   ka:   K fragment addresses of the sub-tile of S^T(u+1), kn: those of the iteration after
+    //         (its first two fragments are read here; the others are computed here from knoff)
+    //   voff: LDS offset of the V sub-tile of P(u-1)
+    //   BAR:  this iteration carries the workgroup barrier, behind which tile T+2 of V and T+4 of
+    //         K are requested into the ring buffers at kld / vld.
+    auto iter = [&](auto bar_c, int (&ka)[KS], int (&kn)[KS], int knoff, int voff, int kld, int vld, int u, int T,
+                    f32x4 (&sc)[2][QB], f32x4 (&sn)[2][QB], uint32_t (&pc)[QB][4], uint32_t (&pp)[QB][4]) {
+        constexpr bool BAR = decltype(bar_c)::value;
+        u32x4 rk, rv;
+        uint32_t m0k = 0, m0v = 0;
+        if constexpr (BAR) {
+            rk = tile_rsrc(kbase, k_row2, (T + 4) * 64);
+            rv = tile_rsrc(vbase, v_row2, (T + 2) * 64);
+            m0k = lds_base + kld;
+            m0v = lds_base + V0 + vld;
+        }
+        bf16x8 ppf[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            const u32x4 v4 = {pp[qb][0], pp[qb][1], pp[qb][2], pp[qb][3]};
+            ppf[qb] = __builtin_bit_cast(bf16x8, v4);
+        }
+        float sum[QB];
+        float e0[2], e1[2];
+        uint64_t trip = 0;
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, 64>([&](auto i_c) {
+            constexpr int i = decltype(i_c)::value;
+            if constexpr (BAR && i == 40) {
+                // V(T), K(T+1) have landed (everything but the newest 12 loads of this wave); every
+                // wave is done with K(T) and V(T-2)
+                attn_vmwait_barrier<12>();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- matrix pipe
+            if constexpr (i < 32) {
+                constexpr int n = i / 4, qb = i % 4, kb = n / 4, ks = n % 4;
+                if constexpr (ks == 0) mfma_s_seed<kAccQ + 16 * qb>(sn[kb][qb], kf[n % 4], seed[qb]);
+                else mfma_s_acc<kAccQ + 16 * qb + 4 * ks>(sn[kb][qb], kf[n % 4]);
+            } else {
+                constexpr int m = (i - 32) / 4, qb = i % 4;
+                mfma_o_acc<16 * m + 4 * qb>(vfrag(m % 4), ppf[qb]);
+            }
+            // ---- LDS addresses of this iteration's V^T fragments and of the next iteration's K fragments
+            if constexpr (i < DBN) va[i] = v_addr[i] + voff;
+            if constexpr (i >= 44 && i < 44 + KS) kn[i - 44] = k_addr[i - 44] + knoff;
+            // ---- LDS fragment reads, eight slots ahead
+            if constexpr (i <= 20 && i % 4 == 0) read_k(ka, i / 4 + 2);
+            if constexpr (i == 56) read_k(kn, 0);
+            if constexpr (i == 60) read_k(kn, 1);
+            if constexpr (i >= 24 && i < 56 && i % 4 == 0) {
+                constexpr int m = (i - 24) / 4;
+                keep_regs(vlo[m % 4]);
+                vlo[m % 4] = lds_read_tr(lds + va[m]);
+            }
+            if constexpr (i >= 24 && i < 56 && i % 4 == 1) {
+                constexpr int m = (i - 25) / 4;
+                keep_regs(vhi[m % 4]);
+                vhi[m % 4] = lds_read_tr(lds + va[m] + 16 * ROWB);
+            }
+            // ---- global loads of later tiles behind the barrier
+            if constexpr (BAR && i > 40 && i <= 56 && i % 2 == 1) {
+                constexpr int j = (i - 41) / 2;
+                if constexpr (j < 4) lds_load16_raw(rv, m0v + j * 4096, v_voff[j]);
+                else lds_load16_raw(rk, m0k + (j - 4) * 4096, k_voff[j - 4]);
+            }
+            // ---- softmax of S^T(u), the steps that belong to this slot
+            static_for<0, attn_step_count(i)>([&](auto jj_c) {
+                constexpr int j = attn_first_step(i) + decltype(jj_c)::value;
+                constexpr int kind = attn_step_kind(j), k = attn_step_unit(j), qb = k / 4, w = k % 4;
+                if constexpr (kind == ATT_E0 || kind == ATT_E1) {
+                    asm volatile("" : "+v"(sc[w / 2][qb]));  // keeps the exponential in its slot
+                    const float a = sc[w / 2][qb][(w % 2) * 2 + (kind == ATT_E1)];
+                    if constexpr (kind == ATT_E0) e0[k % 2] = __builtin_amdgcn_exp2f(a);
+                    else e1[k % 2] = __builtin_amdgcn_exp2f(a);
+                } else if constexpr (kind == ATT_C) {
+                    keep_regs(pc[qb][w]);  // P^T of the iteration before: read by MFMAs a few slots ago
+                    pc[qb][w] = pack2_bf16(e0[k % 2], e1[k % 2]);
+                } else if constexpr (kind == ATT_A0) {
+                    if constexpr (w == 0) sum[qb] = e0[k % 2] + e1[k % 2];
+                    else sum[qb] += e0[k % 2];
+                } else if constexpr (kind == ATT_A1) {
+                    if constexpr (w != 0) sum[qb] += e1[k % 2];
+                } else {
+                    const float big = fmaxf(fmaxf(sum[0], sum[1]), fmaxf(sum[2], sum[3]));
+                    trip = __builtin_amdgcn_ballot_w64(!(big < kRebase));
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // One branch per iteration, off the common path: a reference maximum has to move, or the
+        // next sub-tile reaches past the last key.
+        if (__builtin_expect((trip != 0) | ((u + 2) * 32 > p.L), 0)) {
+            if (trip != 0) rebase(sc, sn, pc, sum);
+            if ((u + 2) * 32 > p.L) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if ((u + 1) * 32 + kb * 16 + g * 4 + j >= p.L) sn[kb][qb][j] = -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) l_run[qb] += sum[qb];
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Body T: iteration 2T (S^T from the second half of K(T), P V with the second half of V(T-1))
+    // and iteration 2T+1 (first half of K(T+1), first half of V(T)). Tile X sits in ring buffer
+    // X % 4. One more body than there are tiles: the last one only finishes P V.
+#ifdef X_CLOCKS
+    const long long x_t1 = clock64();
+#endif
+    for (int T = 0;; ++T) {
+        const int r0 = (T & 3) * TB, r1 = ((T + 1) & 3) * TB, r2 = ((T + 2) & 3) * TB, r3 = ((T + 3) & 3) * TB;
+        iter(std::true_type{}, ka_a, ka_b, r1, r3 + HALF, r0, r2, 2 * T, T, s0, s1, pw0, pw1);
+        if (T == ntiles) break;
+        iter(std::false_type{}, ka_b, ka_a, r1 + HALF, r0, 0, 0, 2 * T + 1, T, s1, s0, pw1, pw0);
+    }
+    wait_all_vmem();
+    mfma_settle();
+#ifdef X_CLOCKS
+    const long long x_t2 = clock64();
+#endif
+
+    // ---- finish: fold the four lane groups' partial sums, normalise, store
+    static_for<0, QB>([&](auto qb_c) {
+        constexpr int qb = decltype(qb_c)::value, QBC = qb;
+        float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
+        l_tot += __shfl_xor(l_tot, 32, 64);
+        const float inv = 1.0f / l_tot;
+        const int row = q0 + qb * 16 + r16;
+        if (row < p.L) {
+            bf16_t* orow = p.o + b * p.o_sb + h * p.o_sh + static_cast<int64_t>(row) * p.o_sl;
+            static_for<0, DBN>([&](auto db_c) {
+                constexpr int db = decltype(db_c)::value, r = 16 * db + 4 * QBC;
+                u32x2 w;
+                w.x = pack2_bf16(acc_read<r>() * inv, acc_read<r + 1>() * inv);
+                w.y = pack2_bf16(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
+                *reinterpret_cast<u32x2*>(orow + db * 16 + g * 4) = w;
+            });
+            if (p.lse != nullptr && g == 0)
+                p.lse[static_cast<int64_t>(bh) * p.L + row] = -seed[qb][0] + __builtin_amdgcn_logf(l_tot);
+        }
+    });
+#ifdef X_CLOCKS
+    if (p.lse != nullptr && tid == 0) {
+        const int64_t at = static_cast<int64_t>(bh) * p.L + qt * 256;
+        p.lse[at] = static_cast<float>(clock64() - x_t0);
+        p.lse[at + 1] = static_cast<float>(wall_clock64() - x_w0);
+        p.lse[at + 2] = static_cast<float>(x_t2 - x_t1);
+        p.lse[at + 3] = static_cast<float>(x_t1 - x_t0);
+    }
+#endif
+}
+
+
 template <int D, int QB, int BN>
 static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
     p.n_qtiles = (p.L + 128 * QB - 1) / (128 * QB);
     p.total_tiles = static_cast<int>(p.n_qtiles * BH);
     const int grid = ((p.total_tiles + 7) / 8) * 8;
     hipLaunchKernelGGL((attn_fwd_pipe_kernel<D, QB, BN>), dim3(grid), dim3(256), 0, st, p);
+}
+
+constexpr int64_t kW64MinTiles = 128;
+
+static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
+    p.n_qtiles = (p.L + 255) / 256;
+    p.total_tiles = static_cast<int>(p.n_qtiles * BH);
+    const int grid = ((p.total_tiles + 7) / 8) * 8;
+    hipLaunchKernelGGL(attn_fwd_w64_kernel, dim3(grid), dim3(256), 0, st, p);
 }
 
 }  // namespace flux
@@ -458,7 +999,7 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     if (!a) return fail(FLUX_E_NULL, "flux_attention_fwd_bf16: null args");
     if (a->B < 0 || a->H <= 0 || a->L < 0) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: bad shape B=%lld H=%lld L=%lld", (long long)a->B, (long long)a->H, (long long)a->L);
     if (a->D != 64 && a->D != 128) return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: head dim %d not supported (64, 128)", a->D);
-    if (!(a->sm_scale >= 0.0f)) return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: sm_scale must be >= 0");
+    if (!(a->sm_scale == a->sm_scale)) return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: sm_scale is NaN");
     if (a->B == 0 || a->L == 0) return FLUX_OK;
     if (a->L > 0x7fffffff / 64 || a->B * a->H > 0x7fffffff / 64) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: problem too large");
     if (!view_ok(a->q.ptr, a->q.sb, a->q.sh, a->q.sl) || !view_ok(a->k.ptr, a->k.sb, a->k.sh, a->k.sl) ||
@@ -477,9 +1018,11 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     p.scale_log2 = a->sm_scale * 1.4426950408889634f;
     const int64_t BH = a->B * a->H;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // One q-block (32 rows) per wave keeps the kernel under 256 registers, so two workgroups share a
-    // CU and each SIMD has a second wave to issue from while the first waits.
-    if (a->D == 128) attn_launch_pipe<128, 1, 64>(p, BH, st);
+    // Head dim 128: 64 rows per wave (256 per workgroup, one workgroup per CU) once there are enough
+    // such tiles to occupy the chip; smaller problems get 128-row workgroups, two per CU.
+    const int64_t tiles256 = BH * ((a->L + 255) / 256);
+    if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64(p, BH, st);
+    else if (a->D == 128) attn_launch_pipe<128, 1, 64>(p, BH, st);
     else attn_launch_pipe<64, 1, 64>(p, BH, st);
     return check_launch("flux_attention_fwd_bf16");
 }
