@@ -78,6 +78,14 @@ __device__ __forceinline__ void lds_load16_raw(u32x4 rsrc, uint32_t lds_addr, ui
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
                  : "memory", "m0");
 }
+// The same with the LDS address given as a scalar base plus a constant.
+template <int OFF>
+__device__ __forceinline__ void lds_load16_raw_at(u32x4 rsrc, uint32_t lds_base, uint32_t voff) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(rsrc), "n"(OFF)
+                 : "memory", "m0", "scc");
+}
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p));
 }
@@ -550,41 +558,80 @@ __device__ __forceinline__ void attn_vmwait_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// VALU work of one iteration as a list of 81 single-instruction steps, spread over the first 60 of
-// the 64 MFMA slots. A unit is two scores of one query block: E0, E1 = their exponentials, C = pack
-// to bf16, A0, A1 = add to the row sum (fp32, from the unrounded values: the dot-product
-// instructions that would sum the rounded pair share the matrix pipe with the MFMAs and cost a
-// whole MFMA slot each). Steps of unit k-1 are interleaved with the exponentials of unit k so that
-// no step waits for the one before it and two exponentials never fall into one slot.
-enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_CHECK };
-constexpr int kAttnSteps = 81;
-constexpr int attn_step_kind(int j) {
-    if (j < 2) return j == 0 ? ATT_E0 : ATT_E1;
-    if (j >= 77) return j == 77 ? ATT_C : j == 78 ? ATT_A0 : j == 79 ? ATT_A1 : ATT_CHECK;
-    constexpr int order[5] = {ATT_E0, ATT_C, ATT_E1, ATT_A0, ATT_A1};
-    return order[(j - 2) % 5];
+// VALU work of one iteration, assigned to the 64 MFMA slots at compile time. A unit is two scores
+// of one query block: E0, E1 = their exponentials, C = pack to bf16, A0, A1 = add to the row sum
+// (fp32, from the unrounded values: the dot-product instructions that would sum the rounded pair
+// run on the matrix pipe and cost a whole MFMA slot each). VA / KN = the LDS addresses of this
+// iteration's V^T fragments and of the next iteration's K fragments (lane part + ring offset).
+// What the schedule is built around, measured on MI355X with one wave per SIMD: beside a 16-cycle
+// MFMA the VALU has room for two ordinary instructions or for one exponential, and an instruction
+// behind an exponential in the same slot waits for it (and so does the next MFMA). So a slot holds
+// either one exponential or up to two other steps; a unit's other steps come two or more slots
+// after its exponentials.
+enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_VA, ATT_KN, ATT_CHECK };
+struct AttnSched {
+    int n[64];
+    int kind[64][6];
+    int arg[64][6];
+};
+constexpr AttnSched attn_sched() {
+    AttnSched S{};
+    int qk[160] = {}, qa[160] = {}, qr[160] = {};  // pending steps: kind, argument, first slot allowed
+    int head = 0, tail = 0, next_exp = 0;
+    for (int m = 0; m < 8; ++m) { qk[tail] = ATT_VA; qa[tail] = m; qr[tail] = 0; ++tail; }
+    for (int s = 0; s < 64; ++s) {
+        const bool exp_slot = s < 4 || s % 2 == 1;
+        if (exp_slot && next_exp < 32) {
+            const int unit = next_exp / 2, second = next_exp % 2;
+            S.kind[s][S.n[s]] = second ? ATT_E1 : ATT_E0; S.arg[s][S.n[s]] = unit; ++S.n[s];
+            if (second) {
+                qk[tail] = ATT_C; qa[tail] = unit; qr[tail] = s + 2; ++tail;
+                qk[tail] = ATT_A0; qa[tail] = unit; qr[tail] = s + 2; ++tail;
+                if (unit % 4 != 0) { qk[tail] = ATT_A1; qa[tail] = unit; qr[tail] = s + 2; ++tail; }
+            }
+            ++next_exp;
+        } else {
+            for (int c = 0; c < 2 && head < tail && qr[head] <= s; ++c) {
+                S.kind[s][S.n[s]] = qk[head]; S.arg[s][S.n[s]] = qa[head]; ++S.n[s]; ++head;
+            }
+        }
+        if (s == 30)
+            for (int k = 0; k < 4; ++k) { qk[tail] = ATT_KN; qa[tail] = k; qr[tail] = 32; ++tail; }
+    }
+    while (head < tail) { S.kind[63][S.n[63]] = qk[head]; S.arg[63][S.n[63]] = qa[head]; ++S.n[63]; ++head; }
+    S.kind[63][S.n[63]] = ATT_CHECK; S.arg[63][S.n[63]] = 0; ++S.n[63];
+    return S;
 }
-constexpr int attn_step_unit(int j) {
-    if (j < 2) return 0;
-    if (j >= 77) return 15;
-    const int k = 1 + (j - 2) / 5, kind = attn_step_kind(j);
-    return (kind == ATT_E0 || kind == ATT_E1) ? k : k - 1;
-}
-constexpr int attn_step_slot(int j) { return j < 2 ? j : 2 + ((j - 2) * 58) / 79; }
-constexpr int attn_first_step(int slot) {  // steps of a slot are consecutive in the list
-    for (int j = 0; j < kAttnSteps; ++j)
-        if (attn_step_slot(j) == slot) return j;
-    return kAttnSteps;
-}
-constexpr int attn_step_count(int slot) {
-    int n = 0;
-    for (int j = 0; j < kAttnSteps; ++j) n += attn_step_slot(j) == slot;
-    return n;
+constexpr bool attn_sched_ok(int la) {  // every step exactly once, addresses ready before their first use
+    const AttnSched S = attn_sched();
+    int seen[8][16] = {};
+    for (int s = 0; s < 64; ++s) {
+        if (S.n[s] > 6) return false;
+        for (int c = 0; c < S.n[s]; ++c) {
+            seen[S.kind[s][c]][S.arg[s][c]] += 1;
+            if (S.kind[s][c] == ATT_VA && s >= 32 + 4 * S.arg[s][c] - la) return false;
+            if (S.kind[s][c] == ATT_KN && (s >= 64 - la || s < 32)) return false;
+        }
+    }
+    for (int u = 0; u < 16; ++u) {
+        if (seen[ATT_E0][u] != 1 || seen[ATT_E1][u] != 1 || seen[ATT_C][u] != 1 || seen[ATT_A0][u] != 1) return false;
+        if (seen[ATT_A1][u] != (u % 4 != 0)) return false;
+    }
+    for (int m = 0; m < 8; ++m) if (seen[ATT_VA][m] != 1) return false;
+    for (int k = 0; k < 4; ++k) if (seen[ATT_KN][k] != 1) return false;
+    return seen[ATT_CHECK][0] == 1;
 }
 
 __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     constexpr int D = 128, QB = 4, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
     constexpr int V0 = 4 * TB;
+#ifndef X_LA
+#define X_LA 12
+#endif
+    constexpr int LA = X_LA;  // look-ahead of the LDS fragment reads, in MFMA slots (a ring of four holds up to 12)
+    static_assert(LA % 4 == 0 && LA >= 4 && LA <= 12, "fragment rings have four entries");
+    constexpr AttnSched SCHED = attn_sched();
+    static_assert(attn_sched_ok(LA), "VALU schedule");
     constexpr float kRebase = 1.0995116e12f;  // 2^40
     __shared__ __attribute__((aligned(1024))) char lds[8 * TB + 4096];  // K ring of 4 tiles, V ring of 4 tiles, 1 KB per wave for the re-base
 
@@ -769,8 +816,8 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) ka_a[ks] = k_addr[ks] + HALF;  // second half of K(0)
     mfma_settle_seeds(seed);
-    read_k(ka_a, 0);
-    read_k(ka_a, 1);
+#pragma unroll
+    for (int n = 0; 4 * n < LA; ++n) read_k(ka_a, n);
     __builtin_amdgcn_sched_barrier(0);
 
     // Shift the reference maxima of all rows of the wave (rare). sc = S^T of the sub-tile whose
@@ -815,18 +862,12 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     //         (its first two fragments are read here; the others are computed here from knoff)
     //   voff: LDS offset of the V sub-tile of P(u-1)
     //   BAR:  this iteration carries the workgroup barrier, behind which tile T+2 of V and T+4 of
-    //         K are requested into the ring buffers at kld / vld.
-    auto iter = [&](auto bar_c, int (&ka)[KS], int (&kn)[KS], int knoff, int voff, int kld, int vld, int u, int T,
+    //         K are requested (descriptors rk / rv, LDS targets m0k / m0v), spread over this
+    //         iteration and the next one.
+    auto iter = [&](auto bar_c, int (&ka)[KS], int (&kn)[KS], int knoff, int voff, const u32x4& rk, const u32x4& rv,
+                    uint32_t m0k, uint32_t m0v, int u,
                     f32x4 (&sc)[2][QB], f32x4 (&sn)[2][QB], uint32_t (&pc)[QB][4], uint32_t (&pp)[QB][4]) {
         constexpr bool BAR = decltype(bar_c)::value;
-        u32x4 rk, rv;
-        uint32_t m0k = 0, m0v = 0;
-        if constexpr (BAR) {
-            rk = tile_rsrc(kbase, k_row2, (T + 4) * 64);
-            rv = tile_rsrc(vbase, v_row2, (T + 2) * 64);
-            m0k = lds_base + kld;
-            m0v = lds_base + V0 + vld;
-        }
         bf16x8 ppf[QB];
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
@@ -834,17 +875,19 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
             ppf[qb] = __builtin_bit_cast(bf16x8, v4);
         }
         float sum[QB];
-        float e0[2], e1[2];
+        float e0[4], e1[4];  // exponentials of up to four units in flight
         uint64_t trip = 0;
         __builtin_amdgcn_sched_barrier(0);
         static_for<0, 64>([&](auto i_c) {
             constexpr int i = decltype(i_c)::value;
+#ifndef X_NOBAR
             if constexpr (BAR && i == 40) {
                 // V(T), K(T+1) have landed (everything but the newest 12 loads of this wave); every
                 // wave is done with K(T) and V(T-2)
                 attn_vmwait_barrier<12>();
                 __builtin_amdgcn_sched_barrier(0);
             }
+#endif
             // ---- matrix pipe
             if constexpr (i < 32) {
                 constexpr int n = i / 4, qb = i % 4, kb = n / 4, ks = n % 4;
@@ -854,46 +897,57 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
                 constexpr int m = (i - 32) / 4, qb = i % 4;
                 mfma_o_acc<16 * m + 4 * qb>(vfrag(m % 4), ppf[qb]);
             }
-            // ---- LDS addresses of this iteration's V^T fragments and of the next iteration's K fragments
-            if constexpr (i < DBN) va[i] = v_addr[i] + voff;
-            if constexpr (i >= 44 && i < 44 + KS) kn[i - 44] = k_addr[i - 44] + knoff;
-            // ---- LDS fragment reads, eight slots ahead
-            if constexpr (i <= 20 && i % 4 == 0) read_k(ka, i / 4 + 2);
-            if constexpr (i == 56) read_k(kn, 0);
-            if constexpr (i == 60) read_k(kn, 1);
-            if constexpr (i >= 24 && i < 56 && i % 4 == 0) {
-                constexpr int m = (i - 24) / 4;
-                keep_regs(vlo[m % 4]);
-                vlo[m % 4] = lds_read_tr(lds + va[m]);
-            }
-            if constexpr (i >= 24 && i < 56 && i % 4 == 1) {
-                constexpr int m = (i - 25) / 4;
-                keep_regs(vhi[m % 4]);
-                vhi[m % 4] = lds_read_tr(lds + va[m] + 16 * ROWB);
-            }
+            // ---- LDS fragment reads, LA slots ahead of the first MFMA that takes them (K fragment n
+            // feeds slots 4n..4n+3, V^T fragment m slots 32+4m..35+4m; the first K fragments of an
+            // iteration are read in the one before)
+#ifndef X_NOLDS
+            static_for<0, 8>([&](auto n_c) {
+                constexpr int n = decltype(n_c)::value;
+                if constexpr (4 * n - LA == i) read_k(ka, n);
+                if constexpr (64 + 4 * n - LA == i) read_k(kn, n);
+                if constexpr (32 + 4 * n - LA == i) {
+                    keep_regs(vlo[n % 4]);
+                    vlo[n % 4] = lds_read_tr(lds + va[n]);
+                }
+                if constexpr (33 + 4 * n - LA == i) {
+                    keep_regs(vhi[n % 4]);
+                    vhi[n % 4] = lds_read_tr(lds + va[n] + 16 * ROWB);
+                }
+            });
+#endif
             // ---- global loads of later tiles behind the barrier
-            if constexpr (BAR && i > 40 && i <= 56 && i % 2 == 1) {
-                constexpr int j = (i - 41) / 2;
-                if constexpr (j < 4) lds_load16_raw(rv, m0v + j * 4096, v_voff[j]);
-                else lds_load16_raw(rk, m0k + (j - 4) * 4096, k_voff[j - 4]);
+#ifndef X_NOLOAD
+            // (eight per tile and wave, one every eight slots: V(T+2) first, then K(T+4))
+            if constexpr (i % 8 == 4 && (BAR ? i > 40 : i < 40)) {
+                constexpr int j = BAR ? (i - 44) / 8 : 3 + (i - 4) / 8;
+                if constexpr (j < 4) lds_load16_raw_at<j * 4096>(rv, m0v, v_voff[j]);
+                else lds_load16_raw_at<(j - 4) * 4096>(rk, m0k, k_voff[j - 4]);
             }
+#endif
             // ---- softmax of S^T(u), the steps that belong to this slot
-            static_for<0, attn_step_count(i)>([&](auto jj_c) {
-                constexpr int j = attn_first_step(i) + decltype(jj_c)::value;
-                constexpr int kind = attn_step_kind(j), k = attn_step_unit(j), qb = k / 4, w = k % 4;
+            // ---- VALU steps of this slot: softmax of S^T(u), LDS addresses
+            static_for<0, SCHED.n[i]>([&](auto c_c) {
+                constexpr int c = decltype(c_c)::value, kind = SCHED.kind[i][c], k = SCHED.arg[i][c], qb = (k / 4) % 4, w = k % 4;
                 if constexpr (kind == ATT_E0 || kind == ATT_E1) {
-                    asm volatile("" : "+v"(sc[w / 2][qb]));  // keeps the exponential in its slot
+                    // issued from asm: it stays in its slot, and the compiler adds no wait state in
+                    // front of it (nothing reads the result before the next slot but one)
                     const float a = sc[w / 2][qb][(w % 2) * 2 + (kind == ATT_E1)];
-                    if constexpr (kind == ATT_E0) e0[k % 2] = __builtin_amdgcn_exp2f(a);
-                    else e1[k % 2] = __builtin_amdgcn_exp2f(a);
+                    float e;
+                    asm volatile("v_exp_f32 %0, %1" : "=v"(e) : "v"(a));
+                    if constexpr (kind == ATT_E0) e0[k % 4] = e;
+                    else e1[k % 4] = e;
                 } else if constexpr (kind == ATT_C) {
                     keep_regs(pc[qb][w]);  // P^T of the iteration before: read by MFMAs a few slots ago
-                    pc[qb][w] = pack2_bf16(e0[k % 2], e1[k % 2]);
+                    pc[qb][w] = pack2_bf16(e0[k % 4], e1[k % 4]);
                 } else if constexpr (kind == ATT_A0) {
-                    if constexpr (w == 0) sum[qb] = e0[k % 2] + e1[k % 2];
-                    else sum[qb] += e0[k % 2];
+                    if constexpr (w == 0) sum[qb] = e0[k % 4] + e1[k % 4];
+                    else sum[qb] += e0[k % 4];
                 } else if constexpr (kind == ATT_A1) {
-                    if constexpr (w != 0) sum[qb] += e1[k % 2];
+                    sum[qb] += e1[k % 4];
+                } else if constexpr (kind == ATT_VA) {
+                    va[k] = v_addr[k] + voff;
+                } else if constexpr (kind == ATT_KN) {
+                    kn[k] = k_addr[k] + knoff;
                 } else {
                     const float big = fmaxf(fmaxf(sum[0], sum[1]), fmaxf(sum[2], sum[3]));
                     trip = __builtin_amdgcn_ballot_w64(!(big < kRebase));
@@ -928,9 +982,11 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
 #endif
     for (int T = 0;; ++T) {
         const int r0 = (T & 3) * TB, r1 = ((T + 1) & 3) * TB, r2 = ((T + 2) & 3) * TB, r3 = ((T + 3) & 3) * TB;
-        iter(std::true_type{}, ka_a, ka_b, r1, r3 + HALF, r0, r2, 2 * T, T, s0, s1, pw0, pw1);
+        const u32x4 rk = tile_rsrc(kbase, k_row2, (T + 4) * 64), rv = tile_rsrc(vbase, v_row2, (T + 2) * 64);
+        const uint32_t m0k = lds_base + r0, m0v = lds_base + V0 + r2;
+        iter(std::true_type{}, ka_a, ka_b, r1, r3 + HALF, rk, rv, m0k, m0v, 2 * T, s0, s1, pw0, pw1);
         if (T == ntiles) break;
-        iter(std::false_type{}, ka_b, ka_a, r1 + HALF, r0, 0, 0, 2 * T + 1, T, s1, s0, pw1, pw0);
+        iter(std::false_type{}, ka_b, ka_a, r1 + HALF, r0, rk, rv, m0k, m0v, 2 * T + 1, s1, s0, pw1, pw0);
     }
     wait_all_vmem();
     mfma_settle();
