@@ -44,6 +44,10 @@ struct AttnParams {
     int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, o_sb, o_sh, o_sl;
     int H, L, n_qtiles, total_tiles;
     float scale_log2;  // sm_scale * log2(e)
+    // 64-row-per-wave kernel only: query rows of a launch. (batch*head) pairs are taken two at a
+    // time; the even one gets cnt_even tiles starting at row first_even, the odd one cnt_odd tiles
+    // from first_odd.
+    int cnt_even, cnt_odd, first_even, first_odd;
 };
 
 constexpr unsigned kAttnRsrcFlags = 0x00020000u;
@@ -498,13 +502,18 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // writes keeps that role for the whole loop (keep_regs in front of each redefinition), so that the
 // compiler cannot hand it to a VALU temporary while an MFMA that uses it is still queued.
 #define ATTN_A16(b) "a" #b "0", "a" #b "1", "a" #b "2", "a" #b "3", "a" #b "4", "a" #b "5", "a" #b "6", "a" #b "7", "a" #b "8", "a" #b "9"
-__device__ __forceinline__ void attn_claim_agprs() {
+template <int N> __device__ __forceinline__ void attn_claim_agprs() {  // a0 .. a(N-1)
+    static_assert(N == 96 || N == 144 || N == 192, "clobber lists are spelled out");
     asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", ATTN_A16(1), ATTN_A16(2), ATTN_A16(3),
-                 ATTN_A16(4), ATTN_A16(5), ATTN_A16(6), ATTN_A16(7), ATTN_A16(8), ATTN_A16(9), ATTN_A16(10), ATTN_A16(11),
-                 ATTN_A16(12), ATTN_A16(13), ATTN_A16(14), ATTN_A16(15), ATTN_A16(16), ATTN_A16(17), ATTN_A16(18), "a190", "a191");
+                 ATTN_A16(4), ATTN_A16(5), ATTN_A16(6), ATTN_A16(7), ATTN_A16(8), "a90", "a91", "a92", "a93", "a94", "a95");
+    if constexpr (N >= 144)
+        asm volatile("" ::: "a96", "a97", "a98", "a99", ATTN_A16(10), ATTN_A16(11), ATTN_A16(12), ATTN_A16(13),
+                     "a140", "a141", "a142", "a143");
+    if constexpr (N == 192)
+        asm volatile("" ::: "a144", "a145", "a146", "a147", "a148", "a149", ATTN_A16(15), ATTN_A16(16), ATTN_A16(17), ATTN_A16(18),
+                     "a190", "a191");
 }
 #undef ATTN_A16
-constexpr int kAccQ = 128;  // first accumulation register of the Q fragments
 // S^T block (vector registers) = K fragment x Q fragment (accumulation registers QLO..QLO+3) + c
 template <int QLO>
 __device__ __forceinline__ void mfma_s_seed(f32x4& d, const bf16x8& a, const f32x4& c) {
@@ -542,15 +551,25 @@ __device__ __forceinline__ void mfma_settle() { asm volatile("s_nop 15\n\ts_nop 
 __device__ __forceinline__ void mfma_settle_seeds(f32x4 (&b)[4]) {
     asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : : "memory");
 }
+__device__ __forceinline__ void mfma_settle_seeds(f32x4 (&b)[3]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]) : : "memory");
+}
+__device__ __forceinline__ void mfma_settle_seeds(f32x4 (&b)[2]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0]), "+v"(b[1]) : : "memory");
+}
 // The same, and the compiler may not move a use of the S^T blocks in b across it (register-only
 // code is otherwise free to float above an asm statement it has no operand in common with).
-template <int QB>
-__device__ __forceinline__ void mfma_settle(f32x4 (&b)[2][QB]) {
-    static_assert(QB == 4, "operand list");
+__device__ __forceinline__ void mfma_settle(f32x4 (&b)[2][4]) {
     asm volatile("s_nop 15\n\ts_nop 15"
                  : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[1][2]), "+v"(b[1][3])
                  :
                  : "memory");
+}
+__device__ __forceinline__ void mfma_settle(f32x4 (&b)[2][3]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[1][2]) : : "memory");
+}
+__device__ __forceinline__ void mfma_settle(f32x4 (&b)[2][2]) {
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]) : : "memory");
 }
 
 template <int N>
@@ -571,17 +590,22 @@ __device__ __forceinline__ void attn_vmwait_barrier() {
 enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_VA, ATT_KN, ATT_CHECK };
 struct AttnSched {
     int n[64];
-    int kind[64][6];
-    int arg[64][6];
+    int kind[64][8];
+    int arg[64][8];
 };
+// QB = 16-row query blocks per wave: 16*QB slots, 4*QB units. With one wave per SIMD (QB = 4) a slot
+// takes one exponential or two other steps; with two waves per SIMD (QB = 2) the other wave fills
+// the gaps, there are fewer slots per step, and three other steps share a slot.
+template <int QB>
 constexpr AttnSched attn_sched() {
+    constexpr int NS = 16 * QB, NE = 8 * QB, PER = QB >= 3 ? 2 : 3;
     AttnSched S{};
     int qk[160] = {}, qa[160] = {}, qr[160] = {};  // pending steps: kind, argument, first slot allowed
     int head = 0, tail = 0, next_exp = 0;
     for (int m = 0; m < 8; ++m) { qk[tail] = ATT_VA; qa[tail] = m; qr[tail] = 0; ++tail; }
-    for (int s = 0; s < 64; ++s) {
+    for (int s = 0; s < NS; ++s) {
         const bool exp_slot = s < 4 || s % 2 == 1;
-        if (exp_slot && next_exp < 32) {
+        if (exp_slot && next_exp < NE) {
             const int unit = next_exp / 2, second = next_exp % 2;
             S.kind[s][S.n[s]] = second ? ATT_E1 : ATT_E0; S.arg[s][S.n[s]] = unit; ++S.n[s];
             if (second) {
@@ -591,29 +615,31 @@ constexpr AttnSched attn_sched() {
             }
             ++next_exp;
         } else {
-            for (int c = 0; c < 2 && head < tail && qr[head] <= s; ++c) {
+            for (int c = 0; c < PER && head < tail && qr[head] <= s; ++c) {
                 S.kind[s][S.n[s]] = qk[head]; S.arg[s][S.n[s]] = qa[head]; ++S.n[s]; ++head;
             }
         }
-        if (s == 30)
-            for (int k = 0; k < 4; ++k) { qk[tail] = ATT_KN; qa[tail] = k; qr[tail] = 32; ++tail; }
+        if (s == NS / 2 - 2)
+            for (int k = 0; k < 4; ++k) { qk[tail] = ATT_KN; qa[tail] = k; qr[tail] = NS / 2; ++tail; }
     }
-    while (head < tail) { S.kind[63][S.n[63]] = qk[head]; S.arg[63][S.n[63]] = qa[head]; ++S.n[63]; ++head; }
-    S.kind[63][S.n[63]] = ATT_CHECK; S.arg[63][S.n[63]] = 0; ++S.n[63];
+    while (head < tail) { S.kind[NS - 1][S.n[NS - 1]] = qk[head]; S.arg[NS - 1][S.n[NS - 1]] = qa[head]; ++S.n[NS - 1]; ++head; }
+    S.kind[NS - 1][S.n[NS - 1]] = ATT_CHECK; S.arg[NS - 1][S.n[NS - 1]] = 0; ++S.n[NS - 1];
     return S;
 }
+template <int QB>
 constexpr bool attn_sched_ok(int la) {  // every step exactly once, addresses ready before their first use
-    const AttnSched S = attn_sched();
+    constexpr int NS = 16 * QB;
+    const AttnSched S = attn_sched<QB>();
     int seen[8][16] = {};
-    for (int s = 0; s < 64; ++s) {
-        if (S.n[s] > 6) return false;
+    for (int s = 0; s < NS; ++s) {
+        if (S.n[s] > 8) return false;
         for (int c = 0; c < S.n[s]; ++c) {
             seen[S.kind[s][c]][S.arg[s][c]] += 1;
-            if (S.kind[s][c] == ATT_VA && s >= 32 + 4 * S.arg[s][c] - la) return false;
-            if (S.kind[s][c] == ATT_KN && (s >= 64 - la || s < 32)) return false;
+            if (S.kind[s][c] == ATT_VA && s >= NS / 2 + QB * S.arg[s][c] - la) return false;
+            if (S.kind[s][c] == ATT_KN && (s >= NS - la || s < NS / 2)) return false;
         }
     }
-    for (int u = 0; u < 16; ++u) {
+    for (int u = 0; u < 4 * QB; ++u) {
         if (seen[ATT_E0][u] != 1 || seen[ATT_E1][u] != 1 || seen[ATT_C][u] != 1 || seen[ATT_A0][u] != 1) return false;
         if (seen[ATT_A1][u] != (u % 4 != 0)) return false;
     }
@@ -621,30 +647,53 @@ constexpr bool attn_sched_ok(int la) {  // every step exactly once, addresses re
     for (int k = 0; k < 4; ++k) if (seen[ATT_KN][k] != 1) return false;
     return seen[ATT_CHECK][0] == 1;
 }
+// Slot of the j-th buffer load of a tile (LPW per wave and tile): behind the barrier (slot BS of the
+// first iteration of a body), SP slots apart, continued in the second iteration up to its slot BS.
+constexpr int attn_load_slot(int j, int ns, int bs, int sp, bool second) {
+    int k = 0;
+    for (int s = bs + sp / 2; s < ns; s += sp, ++k)
+        if (k == j) return second ? -1 : s;
+    for (int s = sp / 2; s < bs; s += sp, ++k)
+        if (k == j) return second ? s : -1;
+    return -2;  // does not fit
+}
 
-__global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
-    constexpr int D = 128, QB = 4, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
+// QB = 16-row query blocks per wave, NW = waves per workgroup: 16*QB*NW query rows per workgroup.
+//   <4, 4>: 64 rows per wave, 256 per workgroup, one wave per SIMD (428 registers).
+//   <3, 4>: 48 rows per wave, 192 per workgroup: the same code with three quarters of the work per
+//           iteration, for the launch that evens out the last round (see attn_launch_w64).
+template <int QB, int NW>
+__global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) {
+    static_assert(NW == 4 && (QB == 3 || QB == 4), "configurations that have been laid out and measured");
+    constexpr int ROWS = 16 * QB * NW;         // query rows per workgroup
+    constexpr int D = 128, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
     constexpr int V0 = 4 * TB;
-#ifndef X_LA
-#define X_LA 12
-#endif
-    constexpr int LA = X_LA;  // look-ahead of the LDS fragment reads, in MFMA slots (a ring of four holds up to 12)
-    static_assert(LA % 4 == 0 && LA >= 4 && LA <= 12, "fragment rings have four entries");
-    constexpr AttnSched SCHED = attn_sched();
-    static_assert(attn_sched_ok(LA), "VALU schedule");
+    constexpr int NS = 16 * QB, NSS = 8 * QB;  // MFMA slots per iteration; the first NSS are S^T
+    constexpr int LA = 3 * QB;                 // look-ahead of the LDS fragment reads in slots: what a ring of four fragments holds
+    constexpr int BS = 10 * QB;                // slot of the barrier in the first iteration of a body
+    constexpr int PP = 16 / NW;                // loader passes per tile and operand (a pass = 4 rows per wave)
+    constexpr int LPW = 2 * PP;                // buffer loads per wave and body: PP of V(T+2), then PP of K(T+4)
+    constexpr int kAccQ = 32 * QB;             // first accumulation register of the Q fragments
+    constexpr AttnSched SCHED = attn_sched<QB>();
+    static_assert(attn_sched_ok<QB>(LA), "VALU schedule");
+    static_assert(BS > 7 * QB - LA && BS < NS - LA, "barrier between the last read of K(T) and the first of K(T+1)");
+    static_assert(attn_load_slot(LPW - 1, NS, BS, NS / 8, false) != -2, "load slots");
     constexpr float kRebase = 1.0995116e12f;  // 2^40
-    __shared__ __attribute__((aligned(1024))) char lds[8 * TB + 4096];  // K ring of 4 tiles, V ring of 4 tiles, 1 KB per wave for the re-base
+    __shared__ __attribute__((aligned(1024))) char lds[8 * TB];  // K ring of 4 tiles, V ring of 4 tiles
 
     const int per_xcd = gridDim.x / 8;
     const int vt = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (vt >= p.total_tiles) return;
-    const int bh = vt / p.n_qtiles, qt = vt % p.n_qtiles;
+    const int per_pair = p.cnt_even + p.cnt_odd;
+    const int pair = vt / per_pair, rem = vt % per_pair;
+    const bool odd = rem >= p.cnt_even;
+    const int bh = 2 * pair + odd, qt = odd ? rem - p.cnt_even : rem;
     const int b = bh / p.H, h = bh % p.H;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
-    const int q0 = qt * 256 + wave * 64;
+    const int q0 = (odd ? p.first_odd : p.first_even) + qt * ROWS + wave * (16 * QB);
     const float c = p.scale_log2;
 #ifdef X_CLOCKS
     const long long x_t0 = clock64(), x_w0 = wall_clock64();
@@ -653,15 +702,15 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
     const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
 
-    // loader: a wave-wide load is 4 rows x 256 bytes; pass i covers rows i*16 + wave*4 + lane/16.
+    // loader: a wave-wide load is 4 rows x 256 bytes; pass i covers rows i*4*NW + wave*4 + lane/16.
     // LDS position pos of row r holds the 16-byte chunk pos ^ (r & 15) of a K row (fragment reads
     // take one chunk of 16 consecutive rows) and chunk pos ^ ((r & 7) << 1) of a V row (transposing
     // reads take 32-byte pieces of 4 consecutive rows in each of four lane groups).
     const int l_row = lane >> 4, l_pos = lane & 15;
-    uint32_t k_voff[4], v_voff[4];
+    uint32_t k_voff[PP], v_voff[PP];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = i * 16 + wave * 4 + l_row;
+    for (int i = 0; i < PP; ++i) {
+        const int r = i * 4 * NW + wave * 4 + l_row;
         k_voff[i] = static_cast<uint32_t>((r * p.k_sl + ((l_pos ^ (r & 15)) * 8)) * 2);
         v_voff[i] = static_cast<uint32_t>((r * p.v_sl + ((l_pos ^ ((r & 7) << 1)) * 8)) * 2);
     }
@@ -678,16 +727,15 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
         return r;
     };
     const uint32_t lds_base = lds_addr_of(lds) + wave * 1024;
-    const uint32_t scr_addr = lds_addr_of(lds) + 8 * TB + tid * 16;
     auto load_k = [&](int tile, int buf) {
         const u32x4 rs = tile_rsrc(kbase, k_row2, tile * 64);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lds_load16_raw(rs, lds_base + buf * TB + i * 4096, k_voff[i]);
+        for (int i = 0; i < PP; ++i) lds_load16_raw(rs, lds_base + buf * TB + i * (NW * 1024), k_voff[i]);
     };
     auto load_v = [&](int tile, int buf) {
         const u32x4 rs = tile_rsrc(vbase, v_row2, tile * 64);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lds_load16_raw(rs, lds_base + V0 + buf * TB + i * 4096, v_voff[i]);
+        for (int i = 0; i < PP; ++i) lds_load16_raw(rs, lds_base + V0 + buf * TB + i * (NW * 1024), v_voff[i]);
     };
 
     // The first pass through the loop multiplies P = 0 with whatever the last V buffer holds:
@@ -695,7 +743,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     {
         const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds + V0 + 3 * TB + i * 4096 + tid * 16) = z;
+        for (int i = 0; i < 16 / NW; ++i) *reinterpret_cast<u32x4*>(lds + V0 + 3 * TB + i * (NW * 1024) + tid * 16) = z;
     }
     load_k(0, 0);
     load_v(0, 0);
@@ -703,7 +751,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
 
     // Q fragments ("B" operand of S^T): lane holds row q0 + qb*16 + r16, d = ks*32 + g*8 .. +8,
     // scaled by sm_scale*log2(e) and rounded to bf16.
-    attn_claim_agprs();
+    attn_claim_agprs<48 * QB>();
     {
         u32x4 qraw[QB][KS];  // all sixteen loads in flight before the first conversion
 #pragma unroll
@@ -722,7 +770,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
             const uint32_t t = qraw[qb][ks][e];
             acc_write<kAccQ + i>(pack2_bf16(__uint_as_float(t << 16) * c, __uint_as_float(t & 0xffff0000u) * c));
         });
-        static_for<0, 128>([&](auto i_c) { acc_write<decltype(i_c)::value>(0u); });  // O^T = 0
+        static_for<0, 32 * QB>([&](auto i_c) { acc_write<decltype(i_c)::value>(0u); });  // O^T = 0
     }
 
     // fragment addresses, lane part (the ring offset of the sub-tile is added once per iteration,
@@ -784,11 +832,11 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     for (int n = 0; n < 8; ++n) {
         const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % 4] + (n / 4) * 16 * ROWB);
         static_for<0, QB>([&](auto qb_c) {
-            constexpr int qb = decltype(qb_c)::value;
-            if (n % 4 == 0) mfma_s_zero<kAccQ + 16 * qb>(s0[n / 4][qb], f);
-            else if (n % 4 == 1) mfma_s_acc<kAccQ + 16 * qb + 4>(s0[n / 4][qb], f);
-            else if (n % 4 == 2) mfma_s_acc<kAccQ + 16 * qb + 8>(s0[n / 4][qb], f);
-            else mfma_s_acc<kAccQ + 16 * qb + 12>(s0[n / 4][qb], f);
+            constexpr int qb = decltype(qb_c)::value, QA = 32 * QB + 16 * qb;
+            if (n % 4 == 0) mfma_s_zero<QA>(s0[n / 4][qb], f);
+            else if (n % 4 == 1) mfma_s_acc<QA + 4>(s0[n / 4][qb], f);
+            else if (n % 4 == 2) mfma_s_acc<QA + 8>(s0[n / 4][qb], f);
+            else mfma_s_acc<QA + 12>(s0[n / 4][qb], f);
         });
     }
     mfma_settle(s0);
@@ -817,7 +865,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     for (int ks = 0; ks < KS; ++ks) ka_a[ks] = k_addr[ks] + HALF;  // second half of K(0)
     mfma_settle_seeds(seed);
 #pragma unroll
-    for (int n = 0; 4 * n < LA; ++n) read_k(ka_a, n);
+    for (int n = 0; QB * n < LA; ++n) read_k(ka_a, n);
     __builtin_amdgcn_sched_barrier(0);
 
     // Shift the reference maxima of all rows of the wave (rare). sc = S^T of the sub-tile whose
@@ -841,7 +889,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
                 sn[kb][qb] -= d;
             }
             static_for<0, DBN * 4>([&](auto i_c) {
-                constexpr int i = decltype(i_c)::value, r = 16 * (i / 4) + 4 * QBC + i % 4;
+                constexpr int i = decltype(i_c)::value, r = 4 * ((i / 4) * QB + QBC) + i % 4;
                 acc_write<r>(__float_as_uint(acc_read<r>() * f));
             });
             float sm = 0.0f;
@@ -878,38 +926,38 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
         float e0[4], e1[4];  // exponentials of up to four units in flight
         uint64_t trip = 0;
         __builtin_amdgcn_sched_barrier(0);
-        static_for<0, 64>([&](auto i_c) {
+        static_for<0, NS>([&](auto i_c) {
             constexpr int i = decltype(i_c)::value;
 #ifndef X_NOBAR
-            if constexpr (BAR && i == 40) {
-                // V(T), K(T+1) have landed (everything but the newest 12 loads of this wave); every
+            if constexpr (BAR && i == BS) {
+                // V(T), K(T+1) have landed (everything but the newest 1.5 tiles' loads of this wave); every
                 // wave is done with K(T) and V(T-2)
-                attn_vmwait_barrier<12>();
+                attn_vmwait_barrier<3 * PP>();
                 __builtin_amdgcn_sched_barrier(0);
             }
 #endif
             // ---- matrix pipe
-            if constexpr (i < 32) {
-                constexpr int n = i / 4, qb = i % 4, kb = n / 4, ks = n % 4;
+            if constexpr (i < NSS) {
+                constexpr int n = i / QB, qb = i % QB, kb = n / 4, ks = n % 4;
                 if constexpr (ks == 0) mfma_s_seed<kAccQ + 16 * qb>(sn[kb][qb], kf[n % 4], seed[qb]);
                 else mfma_s_acc<kAccQ + 16 * qb + 4 * ks>(sn[kb][qb], kf[n % 4]);
             } else {
-                constexpr int m = (i - 32) / 4, qb = i % 4;
-                mfma_o_acc<16 * m + 4 * qb>(vfrag(m % 4), ppf[qb]);
+                constexpr int m = (i - NSS) / QB, qb = i % QB;
+                mfma_o_acc<4 * (m * QB + qb)>(vfrag(m % 4), ppf[qb]);
             }
             // ---- LDS fragment reads, LA slots ahead of the first MFMA that takes them (K fragment n
-            // feeds slots 4n..4n+3, V^T fragment m slots 32+4m..35+4m; the first K fragments of an
-            // iteration are read in the one before)
+            // feeds slots QB*n .. QB*n+QB-1, V^T fragment m slots NSS+QB*m ..; the first K fragments of
+            // an iteration are read in the one before)
 #ifndef X_NOLDS
             static_for<0, 8>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value;
-                if constexpr (4 * n - LA == i) read_k(ka, n);
-                if constexpr (64 + 4 * n - LA == i) read_k(kn, n);
-                if constexpr (32 + 4 * n - LA == i) {
+                if constexpr (QB * n - LA == i) read_k(ka, n);
+                if constexpr (NS + QB * n - LA == i) read_k(kn, n);
+                if constexpr (NSS + QB * n - LA == i) {
                     keep_regs(vlo[n % 4]);
                     vlo[n % 4] = lds_read_tr(lds + va[n]);
                 }
-                if constexpr (33 + 4 * n - LA == i) {
+                if constexpr (NSS + 1 + QB * n - LA == i) {
                     keep_regs(vhi[n % 4]);
                     vhi[n % 4] = lds_read_tr(lds + va[n] + 16 * ROWB);
                 }
@@ -917,17 +965,19 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
 #endif
             // ---- global loads of later tiles behind the barrier
 #ifndef X_NOLOAD
-            // (eight per tile and wave, one every eight slots: V(T+2) first, then K(T+4))
-            if constexpr (i % 8 == 4 && (BAR ? i > 40 : i < 40)) {
-                constexpr int j = BAR ? (i - 44) / 8 : 3 + (i - 4) / 8;
-                if constexpr (j < 4) lds_load16_raw_at<j * 4096>(rv, m0v, v_voff[j]);
-                else lds_load16_raw_at<(j - 4) * 4096>(rk, m0k, k_voff[j - 4]);
-            }
+            // (LPW per tile and wave, NS/8 slots apart: V(T+2) first, then K(T+4))
+            static_for<0, LPW>([&](auto j_c) {
+                constexpr int j = decltype(j_c)::value;
+                if constexpr (attn_load_slot(j, NS, BS, NS / 8, !BAR) == i) {
+                    if constexpr (j < PP) lds_load16_raw_at<j * NW * 1024>(rv, m0v, v_voff[j]);
+                    else lds_load16_raw_at<(j - PP) * NW * 1024>(rk, m0k, k_voff[j - PP]);
+                }
+            });
 #endif
             // ---- softmax of S^T(u), the steps that belong to this slot
             // ---- VALU steps of this slot: softmax of S^T(u), LDS addresses
             static_for<0, SCHED.n[i]>([&](auto c_c) {
-                constexpr int c = decltype(c_c)::value, kind = SCHED.kind[i][c], k = SCHED.arg[i][c], qb = (k / 4) % 4, w = k % 4;
+                constexpr int c = decltype(c_c)::value, kind = SCHED.kind[i][c], k = SCHED.arg[i][c], qb = (k / 4) % QB, w = k % 4;
                 if constexpr (kind == ATT_E0 || kind == ATT_E1) {
                     // issued from asm: it stays in its slot, and the compiler adds no wait state in
                     // front of it (nothing reads the result before the next slot but one)
@@ -949,7 +999,9 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
                 } else if constexpr (kind == ATT_KN) {
                     kn[k] = k_addr[k] + knoff;
                 } else {
-                    const float big = fmaxf(fmaxf(sum[0], sum[1]), fmaxf(sum[2], sum[3]));
+                    float big = fmaxf(sum[0], sum[1]);
+                    if constexpr (QB >= 3) big = fmaxf(big, sum[2]);
+                    if constexpr (QB == 4) big = fmaxf(big, sum[3]);
                     trip = __builtin_amdgcn_ballot_w64(!(big < kRebase));
                 }
             });
@@ -1004,7 +1056,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
         if (row < p.L) {
             bf16_t* orow = p.o + b * p.o_sb + h * p.o_sh + static_cast<int64_t>(row) * p.o_sl;
             static_for<0, DBN>([&](auto db_c) {
-                constexpr int db = decltype(db_c)::value, r = 16 * db + 4 * QBC;
+                constexpr int db = decltype(db_c)::value, r = 4 * (db * QB + QBC);
                 u32x2 w;
                 w.x = pack2_bf16(acc_read<r>() * inv, acc_read<r + 1>() * inv);
                 w.y = pack2_bf16(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
@@ -1016,7 +1068,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel(AttnParams p) {
     });
 #ifdef X_CLOCKS
     if (p.lse != nullptr && tid == 0) {
-        const int64_t at = static_cast<int64_t>(bh) * p.L + qt * 256;
+        const int64_t at = static_cast<int64_t>(bh) * p.L + q0;
         p.lse[at] = static_cast<float>(clock64() - x_t0);
         p.lse[at + 1] = static_cast<float>(wall_clock64() - x_w0);
         p.lse[at + 2] = static_cast<float>(x_t2 - x_t1);
@@ -1036,11 +1088,46 @@ static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
 
 constexpr int64_t kW64MinTiles = 128;
 
-static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
-    p.n_qtiles = (p.L + 255) / 256;
-    p.total_tiles = static_cast<int>(p.n_qtiles * BH);
+// One workgroup per CU, so a launch of more than one round's worth of equal tiles costs whole
+// rounds: 432 tiles of 256 rows on 256 CUs take as long as 512 would. When the work is between one
+// and two rounds it is cut into two launches instead, each at most one round: 256-row tiles for the
+// first rows of every (batch, head), 192-row tiles for the rest, with the cut alternating between
+// even and odd (batch, head) pairs so that both launches come out close to full. 110 592 rows of
+// the Flux shape become 252 + 240 workgroups, 1.75 rounds' worth of time instead of 2.
+constexpr int kAttnCUs = 256;
+
+template <int QB>
+static void attn_launch_w64_part(AttnParams p, int64_t BH, int cnt_even, int cnt_odd, int first_even, int first_odd, hipStream_t st) {
+    p.cnt_even = cnt_even; p.cnt_odd = cnt_odd; p.first_even = first_even; p.first_odd = first_odd;
+    const int64_t pairs = (BH + 1) / 2;
+    p.total_tiles = static_cast<int>(pairs * (cnt_even + cnt_odd));
+    if (p.total_tiles == 0) return;
+    if (BH % 2) p.total_tiles -= cnt_odd;  // the last pair has no odd member: its tiles sit at the very end
     const int grid = ((p.total_tiles + 7) / 8) * 8;
-    hipLaunchKernelGGL(attn_fwd_w64_kernel, dim3(grid), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((attn_fwd_w64_kernel<QB, 4>), dim3(grid), dim3(256), 0, st, p);
+}
+
+static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
+    const int n256 = (p.L + 255) / 256;
+    const int64_t tiles = BH * n256;
+    if (tiles > kAttnCUs && tiles <= 2 * kAttnCUs && BH % 2 == 0) {
+        // the most 256-row tiles (ne + no per pair) such that both launches fit one round
+        const int64_t pairs = BH / 2;
+        int best_ne = -1, best_no = -1;
+        for (int ne = 0; ne <= n256; ++ne)
+            for (int no = ne; no <= n256; ++no) {
+                const int re = p.L - min(p.L, ne * 256), ro = p.L - min(p.L, no * 256);
+                const int64_t w1 = pairs * (ne + no), w2 = pairs * ((re + 191) / 192 + (ro + 191) / 192);
+                if (w1 <= kAttnCUs && w2 <= kAttnCUs && (best_ne < 0 || ne + no > best_ne + best_no)) { best_ne = ne; best_no = no; }
+            }
+        if (best_ne >= 0) {
+            const int fe = min(p.L, best_ne * 256), fo = min(p.L, best_no * 256);
+            attn_launch_w64_part<4>(p, BH, best_ne, best_no, 0, 0, st);
+            attn_launch_w64_part<3>(p, BH, (p.L - fe + 191) / 192, (p.L - fo + 191) / 192, fe, fo, st);
+            return;
+        }
+    }
+    attn_launch_w64_part<4>(p, BH, n256, n256, 0, 0, st);
 }
 
 }  // namespace flux
