@@ -580,14 +580,13 @@ __device__ __forceinline__ void attn_vmwait_barrier() {
 // VALU work of one iteration, assigned to the 64 MFMA slots at compile time. A unit is two scores
 // of one query block: E0, E1 = their exponentials, C = pack to bf16, A0, A1 = add to the row sum
 // (fp32, from the unrounded values: the dot-product instructions that would sum the rounded pair
-// run on the matrix pipe and cost a whole MFMA slot each). VA / KN = the LDS addresses of this
-// iteration's V^T fragments and of the next iteration's K fragments (lane part + ring offset).
+// run on the matrix pipe and cost a whole MFMA slot each).
 // What the schedule is built around, measured on MI355X with one wave per SIMD: beside a 16-cycle
 // MFMA the VALU has room for two ordinary instructions or for one exponential, and an instruction
 // behind an exponential in the same slot waits for it (and so does the next MFMA). So a slot holds
 // either one exponential or up to two other steps; a unit's other steps come two or more slots
 // after its exponentials.
-enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_VA, ATT_KN, ATT_CHECK };
+enum { ATT_E0, ATT_E1, ATT_C, ATT_A0, ATT_A1, ATT_CHECK };
 struct AttnSched {
     int n[64];
     int kind[64][8];
@@ -602,7 +601,6 @@ constexpr AttnSched attn_sched() {
     AttnSched S{};
     int qk[160] = {}, qa[160] = {}, qr[160] = {};  // pending steps: kind, argument, first slot allowed
     int head = 0, tail = 0, next_exp = 0;
-    for (int m = 0; m < 8; ++m) { qk[tail] = ATT_VA; qa[tail] = m; qr[tail] = 0; ++tail; }
     for (int s = 0; s < NS; ++s) {
         const bool exp_slot = s < 4 || s % 2 == 1;
         if (exp_slot && next_exp < NE) {
@@ -619,8 +617,6 @@ constexpr AttnSched attn_sched() {
                 S.kind[s][S.n[s]] = qk[head]; S.arg[s][S.n[s]] = qa[head]; ++S.n[s]; ++head;
             }
         }
-        if (s == NS / 2 - 2)
-            for (int k = 0; k < 4; ++k) { qk[tail] = ATT_KN; qa[tail] = k; qr[tail] = NS / 2; ++tail; }
     }
     while (head < tail) { S.kind[NS - 1][S.n[NS - 1]] = qk[head]; S.arg[NS - 1][S.n[NS - 1]] = qa[head]; ++S.n[NS - 1]; ++head; }
     S.kind[NS - 1][S.n[NS - 1]] = ATT_CHECK; S.arg[NS - 1][S.n[NS - 1]] = 0; ++S.n[NS - 1];
@@ -635,17 +631,13 @@ constexpr bool attn_sched_ok(int la) {  // every step exactly once, addresses re
         if (S.n[s] > 8) return false;
         for (int c = 0; c < S.n[s]; ++c) {
             seen[S.kind[s][c]][S.arg[s][c]] += 1;
-            if (S.kind[s][c] == ATT_VA && s >= NS / 2 + QB * S.arg[s][c] - la) return false;
-            if (S.kind[s][c] == ATT_KN && (s >= NS - la || s < NS / 2)) return false;
         }
     }
     for (int u = 0; u < 4 * QB; ++u) {
         if (seen[ATT_E0][u] != 1 || seen[ATT_E1][u] != 1 || seen[ATT_C][u] != 1 || seen[ATT_A0][u] != 1) return false;
         if (seen[ATT_A1][u] != (u % 4 != 0)) return false;
     }
-    for (int m = 0; m < 8; ++m) if (seen[ATT_VA][m] != 1) return false;
-    for (int k = 0; k < 4; ++k) if (seen[ATT_KN][k] != 1) return false;
-    return seen[ATT_CHECK][0] == 1;
+    return la > 0 && seen[ATT_CHECK][0] == 1;
 }
 // Slot of the j-th buffer load of a tile (LPW per wave and tile): behind the barrier (slot BS of the
 // first iteration of a body), SP slots apart, continued in the second iteration up to its slot BS.
@@ -815,10 +807,9 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
         for (int w = 0; w < 4; ++w) pw0[qb][w] = pw1[qb][w] = 0u;
         s0[0][qb] = s0[1][qb] = s1[0][qb] = s1[1][qb] = zero4;
     }
-    int ka_a[KS], ka_b[KS], va[DBN];  // K fragment addresses of two consecutive sub-tiles, V^T of one
-    auto read_k = [&](const int (&ka)[KS], int n) {  // n-th K fragment of a sub-tile: key block n/4, d step n%4
+    auto read_k = [&](int off, int n) {  // n-th K fragment of the sub-tile at LDS offset off (a constant): key block n/4, d step n%4
         keep_regs(kf[n % 4]);
-        kf[n % 4] = *reinterpret_cast<const bf16x8*>(lds + ka[n % 4] + (n / 4) * 16 * ROWB);
+        kf[n % 4] = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % 4] + (off + (n / 4) * 16 * ROWB));
     };
     auto vfrag = [&](int m) {
         typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -861,11 +852,9 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) s0[kb][qb] -= mx;
     }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) ka_a[ks] = k_addr[ks] + HALF;  // second half of K(0)
     mfma_settle_seeds(seed);
 #pragma unroll
-    for (int n = 0; QB * n < LA; ++n) read_k(ka_a, n);
+    for (int n = 0; QB * n < LA; ++n) read_k(HALF, n);  // second half of K(0)
     __builtin_amdgcn_sched_barrier(0);
 
     // Shift the reference maxima of all rows of the wave (rare). sc = S^T of the sub-tile whose
@@ -906,16 +895,19 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
     };
 
     // One iteration = 64 slots of (MFMA, fragment reads for later slots, VALU steps of the softmax).
-    //   ka:   K fragment addresses of the sub-tile of S^T(u+1), kn: those of the iteration after
-    //         (its first two fragments are read here; the others are computed here from knoff)
-    //   voff: LDS offset of the V sub-tile of P(u-1)
+    //   KC:   LDS offset of the K sub-tile of S^T(u+1), KN: that of the iteration after (its first
+    //         fragments are read here), VC: offset of the V sub-tile of P(u-1) (relative to V0)
     //   BAR:  this iteration carries the workgroup barrier, behind which tile T+2 of V and T+4 of
-    //         K are requested (descriptors rk / rv, LDS targets m0k / m0v), spread over this
-    //         iteration and the next one.
-    auto iter = [&](auto bar_c, int (&ka)[KS], int (&kn)[KS], int knoff, int voff, const u32x4& rk, const u32x4& rv,
-                    uint32_t m0k, uint32_t m0v, int u,
+    //         K are requested (descriptors rk / rv) into the ring buffers at KLD / VLD, spread over
+    //         this iteration and the next one.
+    //   RAG:  the sub-tile after this one may reach past the last key (the common loop is built
+    //         without that test).
+    // All offsets are compile-time constants: the body is unrolled over the four ring positions.
+    auto iter = [&](auto bar_c, auto rag_c, auto kc_c, auto kn_c, auto vc_c, auto kld_c, auto vld_c, const u32x4& rk, const u32x4& rv, int u,
                     f32x4 (&sc)[2][QB], f32x4 (&sn)[2][QB], uint32_t (&pc)[QB][4], uint32_t (&pp)[QB][4]) {
-        constexpr bool BAR = decltype(bar_c)::value;
+        constexpr bool BAR = decltype(bar_c)::value, RAG = decltype(rag_c)::value;
+        constexpr int KC = decltype(kc_c)::value, KN = decltype(kn_c)::value, VC = decltype(vc_c)::value;
+        constexpr int KLD = decltype(kld_c)::value, VLD = decltype(vld_c)::value;
         bf16x8 ppf[QB];
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
@@ -951,15 +943,15 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
 #ifndef X_NOLDS
             static_for<0, 8>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value;
-                if constexpr (QB * n - LA == i) read_k(ka, n);
-                if constexpr (NS + QB * n - LA == i) read_k(kn, n);
+                if constexpr (QB * n - LA == i) read_k(KC, n);
+                if constexpr (NS + QB * n - LA == i) read_k(KN, n);
                 if constexpr (NSS + QB * n - LA == i) {
                     keep_regs(vlo[n % 4]);
-                    vlo[n % 4] = lds_read_tr(lds + va[n]);
+                    vlo[n % 4] = lds_read_tr(lds + v_addr[n] + VC);
                 }
                 if constexpr (NSS + 1 + QB * n - LA == i) {
                     keep_regs(vhi[n % 4]);
-                    vhi[n % 4] = lds_read_tr(lds + va[n] + 16 * ROWB);
+                    vhi[n % 4] = lds_read_tr(lds + v_addr[n] + (VC + 16 * ROWB));
                 }
             });
 #endif
@@ -969,8 +961,8 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
             static_for<0, LPW>([&](auto j_c) {
                 constexpr int j = decltype(j_c)::value;
                 if constexpr (attn_load_slot(j, NS, BS, NS / 8, !BAR) == i) {
-                    if constexpr (j < PP) lds_load16_raw_at<j * NW * 1024>(rv, m0v, v_voff[j]);
-                    else lds_load16_raw_at<(j - PP) * NW * 1024>(rk, m0k, k_voff[j - PP]);
+                    if constexpr (j < PP) lds_load16_raw_at<V0 + VLD + j * NW * 1024>(rv, lds_base, v_voff[j]);
+                    else lds_load16_raw_at<KLD + (j - PP) * NW * 1024>(rk, lds_base, k_voff[j - PP]);
                 }
             });
 #endif
@@ -994,10 +986,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
                     else sum[qb] += e0[k % 4];
                 } else if constexpr (kind == ATT_A1) {
                     sum[qb] += e1[k % 4];
-                } else if constexpr (kind == ATT_VA) {
-                    va[k] = v_addr[k] + voff;
-                } else if constexpr (kind == ATT_KN) {
-                    kn[k] = k_addr[k] + knoff;
                 } else {
                     float big = fmaxf(sum[0], sum[1]);
                     if constexpr (QB >= 3) big = fmaxf(big, sum[2]);
@@ -1009,9 +997,9 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
         });
         // One branch per iteration, off the common path: a reference maximum has to move, or the
         // next sub-tile reaches past the last key.
-        if (__builtin_expect((trip != 0) | ((u + 2) * 32 > p.L), 0)) {
+        if (__builtin_expect((trip != 0) | (RAG && (u + 2) * 32 > p.L), 0)) {
             if (trip != 0) rebase(sc, sn, pc, sum);
-            if ((u + 2) * 32 > p.L) {
+            if (RAG && (u + 2) * 32 > p.L) {
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -1028,17 +1016,55 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
 
     // Body T: iteration 2T (S^T from the second half of K(T), P V with the second half of V(T-1))
     // and iteration 2T+1 (first half of K(T+1), first half of V(T)). Tile X sits in ring buffer
-    // X % 4. One more body than there are tiles: the last one only finishes P V.
+    // X % 4, so four bodies make one trip of the loop. One more body than there are tiles: the last
+    // one only finishes P V. Bodies whose sub-tiles all lie inside the sequence run without the
+    // ragged-tail test; the last few take the variant with it.
+    // Buffer descriptors of the tiles requested by body T: K(T+4) and V(T+2), advanced by one tile
+    // per body; the record count is what is left of the sequence, at most one tile.
+    uint64_t k_at = reinterpret_cast<uint64_t>(kbase) + static_cast<uint64_t>(4 * 64) * k_row2;
+    uint64_t v_at = reinterpret_cast<uint64_t>(vbase) + static_cast<uint64_t>(2 * 64) * v_row2;
+    int k_left = (p.L - 4 * 64 - 1) * k_row2 + D * 2, v_left = (p.L - 2 * 64 - 1) * v_row2 + D * 2;  // bytes up to the end of the last row
+    const int k_tile = 63 * k_row2 + D * 2, v_tile = 63 * v_row2 + D * 2;
+    auto next_rsrc = [&](uint64_t& at, int& left, int step, int tile) -> u32x4 {
+        u32x4 r;
+        r.x = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at));
+        r.y = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at >> 32) & 0xffffu);
+        r.z = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max(min(left, tile), 0)));
+        r.w = kAttnRsrcFlags;
+        at += static_cast<uint64_t>(step);
+        left -= step;
+        return r;
+    };
+    auto body = [&](auto r_c, auto rag_c, int T) -> bool {
+        constexpr int r = decltype(r_c)::value, r0 = r * TB, r1 = ((r + 1) & 3) * TB, r2 = ((r + 2) & 3) * TB, r3 = ((r + 3) & 3) * TB;
+        using ic = std::integral_constant<int, 0>;
+        const u32x4 rk = next_rsrc(k_at, k_left, 64 * k_row2, k_tile), rv = next_rsrc(v_at, v_left, 64 * v_row2, v_tile);
+        iter(std::true_type{}, rag_c, std::integral_constant<int, r0 + HALF>{}, std::integral_constant<int, r1>{},
+             std::integral_constant<int, r3 + HALF>{}, std::integral_constant<int, r0>{}, std::integral_constant<int, r2>{},
+             rk, rv, 2 * T, s0, s1, pw0, pw1);
+        if (decltype(rag_c)::value && T == ntiles) return false;
+        iter(std::false_type{}, rag_c, std::integral_constant<int, r1>{}, std::integral_constant<int, r1 + HALF>{},
+             std::integral_constant<int, r0>{}, std::integral_constant<int, r0>{}, std::integral_constant<int, r2>{},
+             rk, rv, 2 * T + 1, s1, s0, pw1, pw0);
+        return true;
+    };
 #ifdef X_CLOCKS
     const long long x_t1 = clock64();
 #endif
-    for (int T = 0;; ++T) {
-        const int r0 = (T & 3) * TB, r1 = ((T + 1) & 3) * TB, r2 = ((T + 2) & 3) * TB, r3 = ((T + 3) & 3) * TB;
-        const u32x4 rk = tile_rsrc(kbase, k_row2, (T + 4) * 64), rv = tile_rsrc(vbase, v_row2, (T + 2) * 64);
-        const uint32_t m0k = lds_base + r0, m0v = lds_base + V0 + r2;
-        iter(std::true_type{}, ka_a, ka_b, r1, r3 + HALF, rk, rv, m0k, m0v, 2 * T, s0, s1, pw0, pw1);
-        if (T == ntiles) break;
-        iter(std::false_type{}, ka_b, ka_a, r1 + HALF, r0, rk, rv, m0k, m0v, 2 * T + 1, s1, s0, pw1, pw0);
+    // bodies 0 .. n_plain-1 never look past the last key: (2T + 3) * 32 <= L, in whole trips of four
+    const int n_plain = max(0, (p.L / 32 - 1) / 2) & ~3;
+    int T = 0;
+    for (; T < n_plain; T += 4) {
+        body(std::integral_constant<int, 0>{}, std::false_type{}, T);
+        body(std::integral_constant<int, 1>{}, std::false_type{}, T + 1);
+        body(std::integral_constant<int, 2>{}, std::false_type{}, T + 2);
+        body(std::integral_constant<int, 3>{}, std::false_type{}, T + 3);
+    }
+    for (;; T += 4) {
+        if (!body(std::integral_constant<int, 0>{}, std::true_type{}, T)) break;
+        if (!body(std::integral_constant<int, 1>{}, std::true_type{}, T + 1)) break;
+        if (!body(std::integral_constant<int, 2>{}, std::true_type{}, T + 2)) break;
+        if (!body(std::integral_constant<int, 3>{}, std::true_type{}, T + 3)) break;
     }
     wait_all_vmem();
     mfma_settle();
