@@ -77,7 +77,9 @@ def test_attention_strided_views_and_lse():
     ref = oracle.attention_ref_fp32(q, k, v)
     torch.testing.assert_close(out.float(), ref, atol=1e-2, rtol=0)
     assert (buf[..., H * D:] == 0).all()
-    torch.testing.assert_close(lse, oracle.attention_lse_ref(q, k), atol=1e-3, rtol=1e-4)
+    # the kernel rounds q * sm_scale * log2(e) to bf16 once (2^-9 relative per element), which moves a
+    # score by a few 1e-3 in the base-2 domain; lse inherits that
+    torch.testing.assert_close(lse, oracle.attention_lse_ref(q, k), atol=5e-3, rtol=5e-4)
 
 
 def test_attention_head_dim_assert():
