@@ -86,3 +86,41 @@ def test_argument_checks_reject_before_launch():
     qa = nv.QkvPrepArgs()
     qa.B, qa.H, qa.Lt, qa.Li, qa.D = 1, 0, 0, 4, 128
     assert lib.flux_qkv_prep(ctypes.byref(qa), None) == -2
+
+
+# ---- generated-code check of the attention kernel (see csrc/check_attention_isa.py) ----------------
+def _isa_checker():
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "triton-kernels_amd", "csrc", "check_attention_isa.py")
+    spec = importlib.util.spec_from_file_location("check_attention_isa", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_attention_isa_checker_flags_what_it_should(tmp_path):
+    chk = _isa_checker()
+    good = "\n".join([
+        "_ZN4flux19attn_fwd_w64_kernelILi4ELi4EEEvNS_10AttnParamsE:",
+        "\tv_add_f32_e32 v1, v2, v3",
+        "\t;;#ASMSTART", "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[4:7], v[8:11], a[0:3]", "\t;;#ASMEND",
+        "\ts_endpgm"])
+    f = tmp_path / "good.s"
+    f.write_text(good)
+    assert chk.check(str(f)) == []
+    for bad_line in ("\tv_accvgpr_write_b32 a5, v1", "\tscratch_store_dword off, v1, off offset:4", "\tds_read_b128 a[4:7], v1"):
+        f = tmp_path / "bad.s"
+        f.write_text(good.replace("\tv_add_f32_e32 v1, v2, v3", bad_line))
+        assert len(chk.check(str(f))) == 1, bad_line
+    f = tmp_path / "none.s"
+    f.write_text("_Zother:\n\ts_endpgm\n")
+    assert chk.check(str(f))  # no instantiation found is an error too
+
+
+def test_attention_generated_code_uses_no_accumulation_registers_of_its_own():
+    """The assembly the build keeps must pass the check (build() makes it; skipped when not built)."""
+    import pytest
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "build", "csrc", "attention-hip-amdgcn-amd-amdhsa-gfx950.s")
+    if not os.path.exists(path):
+        pytest.skip("library not built in this tree")
+    assert _isa_checker().check(path) == []

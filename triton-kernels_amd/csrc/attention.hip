@@ -80,7 +80,7 @@ __device__ __forceinline__ void lds_load16_raw(u32x4 rsrc, uint32_t lds_addr, ui
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
-                 : "memory", "m0");
+                 : "memory");  // m0 is written: a register the compiler reserves and never allocates on this target
 }
 // The same with the LDS address given as a scalar base plus a constant.
 template <int OFF>
@@ -88,7 +88,7 @@ __device__ __forceinline__ void lds_load16_raw_at(u32x4 rsrc, uint32_t lds_base,
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_base), "v"(voff), "s"(rsrc), "n"(OFF)
-                 : "memory", "m0", "scc");
+                 : "memory", "scc");  // and m0, see above
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p));
@@ -687,9 +687,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
     const int r16 = lane & 15, g = lane >> 4;
     const int q0 = (odd ? p.first_odd : p.first_even) + qt * ROWS + wave * (16 * QB);
     const float c = p.scale_log2;
-#ifdef X_CLOCKS
-    const long long x_t0 = clock64(), x_w0 = wall_clock64();
-#endif
 
     const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
     const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
@@ -920,14 +917,12 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
         __builtin_amdgcn_sched_barrier(0);
         static_for<0, NS>([&](auto i_c) {
             constexpr int i = decltype(i_c)::value;
-#ifndef X_NOBAR
             if constexpr (BAR && i == BS) {
                 // V(T), K(T+1) have landed (everything but the newest 1.5 tiles' loads of this wave); every
                 // wave is done with K(T) and V(T-2)
                 attn_vmwait_barrier<3 * PP>();
                 __builtin_amdgcn_sched_barrier(0);
             }
-#endif
             // ---- matrix pipe
             if constexpr (i < NSS) {
                 constexpr int n = i / QB, qb = i % QB, kb = n / 4, ks = n % 4;
@@ -940,7 +935,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
             // ---- LDS fragment reads, LA slots ahead of the first MFMA that takes them (K fragment n
             // feeds slots QB*n .. QB*n+QB-1, V^T fragment m slots NSS+QB*m ..; the first K fragments of
             // an iteration are read in the one before)
-#ifndef X_NOLDS
             static_for<0, 8>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value;
                 if constexpr (QB * n - LA == i) read_k(KC, n);
@@ -954,9 +948,7 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
                     vhi[n % 4] = lds_read_tr(lds + v_addr[n] + (VC + 16 * ROWB));
                 }
             });
-#endif
             // ---- global loads of later tiles behind the barrier
-#ifndef X_NOLOAD
             // (LPW per tile and wave, NS/8 slots apart: V(T+2) first, then K(T+4))
             static_for<0, LPW>([&](auto j_c) {
                 constexpr int j = decltype(j_c)::value;
@@ -965,7 +957,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
                     else lds_load16_raw_at<KLD + (j - PP) * NW * 1024>(rk, lds_base, k_voff[j - PP]);
                 }
             });
-#endif
             // ---- softmax of S^T(u), the steps that belong to this slot
             // ---- VALU steps of this slot: softmax of S^T(u), LDS addresses
             static_for<0, SCHED.n[i]>([&](auto c_c) {
@@ -1048,9 +1039,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
              rk, rv, 2 * T + 1, s1, s0, pw1, pw0);
         return true;
     };
-#ifdef X_CLOCKS
-    const long long x_t1 = clock64();
-#endif
     // bodies 0 .. n_plain-1 never look past the last key: (2T + 3) * 32 <= L, in whole trips of four
     const int n_plain = max(0, (p.L / 32 - 1) / 2) & ~3;
     int T = 0;
@@ -1068,9 +1056,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
     }
     wait_all_vmem();
     mfma_settle();
-#ifdef X_CLOCKS
-    const long long x_t2 = clock64();
-#endif
 
     // ---- finish: fold the four lane groups' partial sums, normalise, store
     static_for<0, QB>([&](auto qb_c) {
@@ -1092,15 +1077,6 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
                 p.lse[static_cast<int64_t>(bh) * p.L + row] = -seed[qb][0] + __builtin_amdgcn_logf(l_tot);
         }
     });
-#ifdef X_CLOCKS
-    if (p.lse != nullptr && tid == 0) {
-        const int64_t at = static_cast<int64_t>(bh) * p.L + q0;
-        p.lse[at] = static_cast<float>(clock64() - x_t0);
-        p.lse[at + 1] = static_cast<float>(wall_clock64() - x_w0);
-        p.lse[at + 2] = static_cast<float>(x_t2 - x_t1);
-        p.lse[at + 3] = static_cast<float>(x_t1 - x_t0);
-    }
-#endif
 }
 
 
