@@ -58,11 +58,16 @@ __global__ __launch_bounds__(kPrepBlock) void qkv_prep_kernel(PrepParams p) {
     constexpr int HG = ITER == 1 ? kHeadGroup : 1;        // long rows already give a thread enough loads in flight
     static_assert(G * ITER * VEC == D, "head dim must be a multiple of the vector width");
     const int lane = threadIdx.x % G;
-    // the head group is the fastest-moving block coordinate: blocks in flight together read whole
-    // source rows (all heads of a position are adjacent in a fused qkv projection)
+    // Consecutive workgroup ids go round the eight XCDs, each with an L2 of its own. The grid is a
+    // multiple of eight and XCD x takes the x-th contiguous eighth of the virtual block order, in
+    // which the head group moves fastest: all head groups of a stretch of positions run on one XCD,
+    // whose L2 then fetches those positions' pe rows (and a fused projection's source rows) once.
     const int64_t groups = (p.H + HG - 1) / HG;
-    const int64_t pos_raw = static_cast<int64_t>(blockIdx.x / groups) * ROWS + threadIdx.x / G;
-    const int64_t b = blockIdx.y, h0 = (blockIdx.x % groups) * HG;
+    const int64_t per_xcd = gridDim.x / 8;
+    const int64_t vb = static_cast<int64_t>(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (vb >= groups * ((p.L + ROWS - 1) / ROWS)) return;   // padding blocks of the rounded-up grid
+    const int64_t pos_raw = (vb / groups) * ROWS + threadIdx.x / G;
+    const int64_t b = blockIdx.y, h0 = (vb % groups) * HG;
     const bool ok = pos_raw < p.L;
     const int64_t pos = ok ? pos_raw : p.L - 1;
     const bool is_txt = pos < p.Lt;
@@ -254,8 +259,8 @@ static int prep_launch(const flux_qkv_prep_args& a, hipStream_t st) {
     // rows of one 16-byte vector per lane are walked kHeadGroup heads at a time (see the kernel)
     const int64_t hg = (D / VEC <= 64) ? kHeadGroup : 1;
     const int64_t pos_blocks = (L + rows_per_block - 1) / rows_per_block, groups = (a.H + hg - 1) / hg;
-    if (a.B > 65535 || pos_blocks * groups > 0x7fffffffLL) return fail(FLUX_E_SHAPE, "flux_qkv_prep: grid too large (B=%lld, L=%lld, H=%lld)", (long long)a.B, (long long)L, (long long)a.H);
-    dim3 grid((unsigned)(pos_blocks * groups), (unsigned)a.B);
+    if (a.B > 65535 || pos_blocks * groups > 0x7ffffff0LL) return fail(FLUX_E_SHAPE, "flux_qkv_prep: grid too large (B=%lld, L=%lld, H=%lld)", (long long)a.B, (long long)L, (long long)a.H);
+    dim3 grid((unsigned)((pos_blocks * groups + 7) / 8 * 8), (unsigned)a.B);   // the kernel deals blocks out by XCD
 
 #define LAUNCH(D_, N_, R_) hipLaunchKernelGGL((qkv_prep_kernel<T, TS, D_, N_, R_>), grid, dim3(kPrepBlock), 0, st, p)
 #define BY_FLAGS(D_)                                   \

@@ -155,6 +155,10 @@ class SingleStreamBlock(nn.Module):
     # QKNorm + RoPE inside linear1's epilogue when the shapes allow (heads of 128, sequence length a
     # multiple of 256); otherwise, or with this switched off, one preparation kernel behind linear1
     fuse_qk_epilogue = True
+    # Optional callable(stage, edge), invoked on the launching thread right before (edge "begin") and
+    # right after ("end") the launch of a stage of the fused forward: "linear1", "attention",
+    # "linear2". Benchmarks set it to record stream events around a kernel inside real block passes.
+    stage_hook = None
 
     def __init__(self, hidden_size: int, num_heads: int, mlp_ratio: float = 4.0, qk_scale: float | None = None):
         super().__init__()
@@ -191,6 +195,8 @@ class SingleStreamBlock(nn.Module):
         both = torch.empty((B, L, hid + self.mlp_hidden_dim), dtype=x.dtype, device=x.device)
         both2 = both.view(M, -1)
         _, _, v_src = _heads(qkv, H)
+        hook = self.stage_hook or (lambda stage, edge: None)
+        hook("linear1", "begin")
         pe_ok = pe.dtype == torch.float32 and pe.is_contiguous() and pe.numel() in (L * D * 2, B * L * D * 2)
         if self.fuse_qk_epilogue and pe_ok and qk_fusable(x_mod, self.linear1.weight, L, D):
             # linear1: q and k columns -> bias, RMSNorm, RoPE -> q, k [B,H,L,D]; v columns -> qkv;
@@ -208,12 +214,17 @@ class SingleStreamBlock(nn.Module):
             q_src, k_src, _ = _heads(qkv, H)
             q, k, _ = qkv_prep(q_src, k_src, None, pe=pe,
                                q_scale_img=self.norm.query_norm.scale, k_scale_img=self.norm.key_norm.scale)
+        hook("linear1", "end")
         # attention output lands in both[:, :hid] in "B L (H D)" order
         attn_out = both[..., :hid].view(B, L, H, D).permute(0, 2, 1, 3)
+        hook("attention", "begin")
         attention_into(q, k, v_src, attn_out)
+        hook("attention", "end")
         out = torch.empty_like(x)
+        hook("linear2", "begin")
         linear_into(both2, self.linear2.weight, self.linear2.bias, out=out.view(M, hid),
                     resid=x.contiguous().view(M, hid), gate=mod.gate)
+        hook("linear2", "end")
         return out
 
 
