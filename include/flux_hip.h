@@ -6,8 +6,8 @@
  * stands in for (paths relative to the reference repository root).
  *
  * Conventions
- *   - All data pointers are device pointers. The library never allocates, frees or keeps them
- *     (the one exception is declared at the bottom of this file and says so).
+ *   - All data pointers are device pointers. The library never allocates, frees or keeps them,
+ *     and no kernel uses device memory beyond the buffers its caller passes.
  *   - Strides are in ELEMENTS, not bytes. The innermost dimension is always contiguous.
  *   - `stream` is a hipStream_t passed as void*; work is enqueued on it and never synchronised.
  *   - Return value: 0 = launched; negative = argument rejected before any launch (FLUX_E_*);
@@ -173,9 +173,14 @@ int flux_linear_bf16(const flux_linear_args* args, void* stream);
 /* ---------------------------------------------------------------------------------------------
  * Non-causal attention forward: O = softmax(Q K^T * sm_scale) V, bf16 in/out, fp32 online softmax.
  * Replaces scaled_dot_product_attention / _attn_fwd (kernels/attention.py:173-221, 70-170).
- * q,k,v,o are [B,H,L,D] views with element strides (sb,sh,sl,1) each; D in {64,128}; any L
- * (ragged tails are masked, which the reference does not do). lse (nullable) receives
+ * q,k,v,o are [B,H,L,D] views with element strides (sb,sh,sl,1) each; D in {16,32,64,128,256}
+ * (the set kernels/attention.py:184 accepts); any L (ragged tails are masked, which the reference
+ * does not do); any finite sm_scale, negative and zero included. lse (nullable) receives
  * m + log2(l) per row as fp32 [B,H,L], the quantity kernels/attention.py:166-169 stores.
+ * For D = 64 and 128 the kernels fold sm_scale * log2(e) into Q and round the result to bf16 once
+ * where kernels/attention.py:29-30 scales the fp32 scores: scores, and with them lse, carry that
+ * rounding (a few 1e-3 in the base-2 domain for unit-variance inputs; o stays within 2e-2 of the
+ * fp32 result). D = 16, 32 and 256 run a plain, unpipelined kernel that scales the fp32 scores.
  * ------------------------------------------------------------------------------------------- */
 typedef struct flux_attn_args {
     flux_src4 q, k, v;

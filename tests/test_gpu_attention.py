@@ -86,3 +86,107 @@ def test_attention_head_dim_assert():
     q = torch.zeros(1, 1, 8, 48, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(AssertionError):
         tk.scaled_dot_product_attention(q, q, q)
+
+
+@pytest.mark.parametrize("seq_len", [1, 31, 77, 256, 333, 1024])
+@pytest.mark.parametrize("head_dim", [16, 32, 256])
+def test_attention_other_head_dims(seq_len, head_dim):
+    """The remaining head dims kernels/attention.py:184 accepts; these score in fp32 (no rounding of a
+    pre-scaled q), so lse is held to a tight bound."""
+    g = seeded(seq_len * 3 + head_dim)
+    B, H = 2, 3
+    q, k, v = (randn(g, B, H, seq_len, head_dim, dtype=torch.bfloat16).to(DEV) for _ in range(3))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, seq_len, dtype=torch.float32, device=DEV)
+    tk.attention_into(q, k, v, o, lse=lse)
+    torch.testing.assert_close(o.float(), oracle.attention_ref_fp32(q, k, v), atol=1e-2, rtol=0)
+    torch.testing.assert_close(lse, oracle.attention_lse_ref(q, k), atol=1e-4, rtol=1e-5)
+    if seq_len % 64 == 0:
+        torch.testing.assert_close(tk.scaled_dot_product_attention(q, k, v), oracle.attention_ref(q, k, v), atol=1e-2, rtol=0)
+    # strided source and destination, explicit scale
+    qkv = randn(g, B, seq_len, 3 * H * head_dim, dtype=torch.bfloat16).to(DEV)
+    q2, k2, v2 = oracle.split_heads_ref(qkv, H)
+    out = torch.empty(B, seq_len, H, head_dim, dtype=torch.bfloat16, device=DEV).permute(0, 2, 1, 3)
+    tk.attention_into(q2, k2, v2, out, sm_scale=0.2)
+    torch.testing.assert_close(out.float(), oracle.attention_ref_fp32(q2, k2, v2, 0.2), atol=1e-2, rtol=0)
+
+
+def _prescaled_ref(q, k, v, sm_scale):
+    """What the head-dim-64/128 kernels evaluate: q * sm_scale * log2(e) rounded to bf16 once, scores and
+    softmax in the base-2 domain. Large scores make that one rounding visible, so the cases that
+    drive the scores up are compared with this form (fp32 otherwise)."""
+    q2 = (q.float() * (sm_scale * math.log2(math.e))).bfloat16().float()
+    s = torch.einsum("bhqd,bhkd->bhqk", q2, k.float()) * math.log(2.0)
+    return torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, dim=-1), v.float()), torch.logsumexp(s, -1) * math.log2(math.e)
+
+
+# (batch, heads, seq): which launch shape the head-dim-128 dispatch picks for them
+_WIDE = [(4, 24, 512),    # 64-row-per-wave kernel, one launch of 256-row tiles
+         (4, 24, 1000),   # the same with a ragged last tile
+         (1, 24, 4336),   # two launches (256- and 192-row tiles), ragged
+         (3, 24, 1536),   # two launches, odd batch * even heads
+         (8, 24, 31),     # one partial tile per head
+         (6, 24, 97),
+         (1, 8, 4100)]    # few heads, long ragged sequence
+
+
+@pytest.mark.parametrize("B,H,L", _WIDE)
+def test_attention_wide_tile_launch_shapes(B, H, L):
+    g = seeded(B * 1000 + H * 100 + L)
+    q, k, v = (randn(g, B, H, L, 128, dtype=torch.bfloat16).to(DEV) for _ in range(3))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, L, dtype=torch.float32, device=DEV)
+    tk.attention_into(q, k, v, o, lse=lse)
+    assert torch.isfinite(o.float()).all()
+    for b in range(B):
+        torch.testing.assert_close(o[b:b + 1].float(), oracle.attention_ref_fp32(q[b:b + 1], k[b:b + 1], v[b:b + 1]), atol=1e-2, rtol=0)
+        torch.testing.assert_close(lse[b:b + 1], oracle.attention_lse_ref(q[b:b + 1], k[b:b + 1]), atol=5e-3, rtol=5e-4)
+
+
+@pytest.mark.parametrize("H", [24, 4])   # 24 heads: 64-row-per-wave kernel; 4 heads: 128-row workgroups
+@pytest.mark.parametrize("kind", ["hot", "ramp"])
+def test_attention_large_scores_move_the_reference_maximum(H, kind):
+    """Scores far above the first tile's maximum: the kernels subtract a per-row reference value that is
+    only raised when a partial sum grows too large, and this drives them through that step."""
+    g = seeded(H + len(kind))
+    L = 2048
+    q = (randn(g, 1, H, L, 128) * (30.0 if kind == "hot" else 4.0)).bfloat16().to(DEV)
+    k = randn(g, 1, H, L, 128, dtype=torch.bfloat16).to(DEV)
+    v = randn(g, 1, H, L, 128, dtype=torch.bfloat16).to(DEV)
+    if kind == "ramp":   # later keys score ever higher than earlier ones
+        ramp = torch.linspace(0, 6.0, L, device=DEV).view(1, 1, L, 1)
+        k = (k.float() + ramp * q.float().mean(dim=2, keepdim=True).sign()).bfloat16()
+    sc = 1 / math.sqrt(128)
+    o = torch.empty_like(q)
+    lse = torch.empty(1, H, L, dtype=torch.float32, device=DEV)
+    tk.attention_into(q, k, v, o, sm_scale=sc, lse=lse)
+    ref, lref = _prescaled_ref(q, k, v, sc)
+    assert torch.isfinite(o.float()).all()
+    # nearly one-hot rows: the output is a v value of size up to ~4, where one bf16 ulp is 0.03
+    torch.testing.assert_close(o.float(), ref, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse, lref, atol=2e-2, rtol=1e-4)
+
+
+@pytest.mark.parametrize("B,H,L,D", [(4, 24, 300, 128), (2, 3, 300, 128), (2, 3, 300, 64), (2, 3, 300, 32)])
+@pytest.mark.parametrize("sm_scale", [-0.11, 0.0])
+def test_attention_any_scale_sign(B, H, L, D, sm_scale):
+    """kernels/attention.py:173 takes whatever scale it is given; zero makes every row the mean of v."""
+    g = seeded(B + H + L + D)
+    q, k, v = (randn(g, B, H, L, D, dtype=torch.bfloat16).to(DEV) for _ in range(3))
+    o = tk.scaled_dot_product_attention(q, k, v, sm_scale=sm_scale)
+    torch.testing.assert_close(o.float(), oracle.attention_ref_fp32(q, k, v, sm_scale), atol=1e-2, rtol=0)
+    if sm_scale == 0.0:
+        torch.testing.assert_close(o.float(), v.float().mean(dim=2, keepdim=True).expand_as(o), atol=4e-3, rtol=0)
+
+
+def test_attention_lse_at_the_flux_shape():
+    q, k, v = cfg.config5_attention(DEV)
+    o = torch.empty_like(q)
+    lse = torch.empty(q.shape[:3], dtype=torch.float32, device=DEV)
+    tk.attention_into(q, k, v, o, lse=lse)
+    torch.testing.assert_close(lse, oracle.attention_lse_ref(q, k), atol=5e-3, rtol=5e-4)
+    # o and lse are consistent: exp2(s_ij * log2e - lse_i) sums to one over j, checked on a few rows
+    rows = torch.tensor([0, 255, 256, 3071, 4415, 4607], device=DEV)
+    s = torch.einsum("bhqd,bhkd->bhqk", q[:, :, rows].float(), k.float()) * (math.log2(math.e) / math.sqrt(q.shape[-1]))
+    total = torch.exp2(s - lse[:, :, rows, None]).sum(-1)
+    torch.testing.assert_close(total, torch.ones_like(total), atol=5e-3, rtol=0)

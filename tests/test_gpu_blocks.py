@@ -16,6 +16,17 @@ HEADS, HEAD_DIM = 24, 128
 HID = HEADS * HEAD_DIM
 
 
+def _close(got, want, atol=0.1, mean=6e-3):
+    """The reference's own bound (tests/test_blocks.py: atol 0.1 on outputs of size ~1) catches gross
+    errors only; a wrong rounding site or epilogue shows in the mean error, which for two correct bf16
+    evaluations of a block stays at a few 1e-3."""
+    torch.testing.assert_close(got, want, atol=atol, rtol=0)
+    err = (got.float() - want.float()).abs()
+    assert err.mean().item() < mean, f"mean error {err.mean().item()}"
+    rel = err.pow(2).sum().sqrt() / want.float().pow(2).sum().sqrt()
+    assert rel.item() < 1e-2, f"relative error {rel.item()}"
+
+
 def _pair(kind, seed):
     torch.manual_seed(seed)
     if kind == "single":
@@ -43,11 +54,11 @@ def test_single_stream_block(batch_size, seq_len):
         y_prep = hip(x=x, vec=vec, pe=pe)             # fused, QKNorm + RoPE as one kernel behind linear1
         hip.fused = False
         y_unfused = hip(x=x, vec=vec, pe=pe)
-    torch.testing.assert_close(y_hip, y_ref, atol=0.1, rtol=0)
-    torch.testing.assert_close(y_prep, y_ref, atol=0.1, rtol=0)
-    torch.testing.assert_close(y_unfused, y_ref, atol=0.1, rtol=0)
-    torch.testing.assert_close(y_hip, y_unfused, atol=0.05, rtol=0)
-    torch.testing.assert_close(y_hip, y_prep, atol=0.05, rtol=0)
+    _close(y_hip, y_ref)
+    _close(y_prep, y_ref)
+    _close(y_unfused, y_ref)
+    _close(y_hip, y_unfused, atol=0.05)
+    _close(y_hip, y_prep, atol=0.05)
 
 
 @pytest.mark.parametrize("batch_size", [1, 2])
@@ -71,10 +82,12 @@ def test_double_stream_block(batch_size, img_seq_len):
         assert torch.equal(s_img, h_img) and torch.equal(s_txt, h_txt)
         hip.fused = False
         u_img, u_txt = hip(img=img, txt=txt, vec=vec, pe=pe)
-    torch.testing.assert_close(h_img, r_img, atol=0.1, rtol=0)
-    torch.testing.assert_close(h_txt, r_txt, atol=0.1, rtol=0)
-    torch.testing.assert_close(u_img, r_img, atol=0.1, rtol=0)
-    torch.testing.assert_close(u_txt, r_txt, atol=0.1, rtol=0)
+    _close(h_img, r_img)
+    _close(h_txt, r_txt)
+    _close(u_img, r_img)
+    _close(u_txt, r_txt)
+    _close(h_img, u_img, atol=0.05)
+    _close(h_txt, u_txt, atol=0.05)
 
 
 def test_single_block_4608_tokens_vs_oracle():

@@ -59,3 +59,45 @@ def test_triton_linear_bias_suffix():
                             GROUP_M=8, EVEN_K=True, ALLOW_TF32=False, ACC_TYPE=None, B_PROLOGUE_CAST_TYPE=None,
                             BLOCK_M=128, BLOCK_N=128, BLOCK_K=32)
     torch.testing.assert_close(out.float(), oracle.linear_ref_fp32(a, w, c), atol=2e-2, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,n,ld", [(1, 8, 8), (5, 384, 384), (300, 1024, 1280), (4608, 12288, 21504), (7, 100, 333)])
+def test_gelu_tanh_strided_rows(dtype, rows, n, ld):
+    """flux_gelu_tanh on a [rows, n] view of wider rows: nn.GELU(approximate="tanh") on the mlp half
+    of linear1's output (modules/blocks.py:107,122)."""
+    from triton_kernels.modules.blocks import _gelu_tanh
+    if dtype == torch.float32 and rows * ld > 2 ** 24:
+        pytest.skip("bf16 covers the full-size case")
+    wide = randn(seeded(rows + n), rows, ld, dtype=dtype, std=2.0).to(DEV)
+    x = wide[:, ld - n:]
+    assert x.is_contiguous() == (ld == n or rows == 1)
+    y = _gelu_tanh(x)
+    assert y.is_contiguous() and y.shape == x.shape
+    ref = oracle.gelu_tanh_ref(x.float())
+    if dtype == torch.float32:
+        torch.testing.assert_close(y, ref, atol=2e-6, rtol=1e-5)
+    else:
+        assert ((y.float() - ref).abs() <= ref.abs() * 2.0 ** -8 * 1.01 + 1e-6).all()   # one rounding of the fp32 value
+    # a 3-d view, as the block passes it
+    if rows % 5 == 0:
+        x3 = wide.view(5, rows // 5, ld)[..., ld - n:]
+        assert torch.equal(_gelu_tanh(x3).view(rows, n), y)
+
+
+@pytest.mark.parametrize("B,L,hid", [(1, 4608, 3072), (2, 77, 384), (3, 1, 8)])
+def test_gated_residual_rounds_the_product(B, L, hid):
+    """flux_gate_residual with round_product = 1: exactly what the two PyTorch ops x + gate * y of
+    modules/blocks.py:123,166-171 produce in bf16 (product rounded, then the sum rounded)."""
+    from triton_kernels.modules.blocks import _gated_residual
+    g = seeded(B + L + hid)
+    x = randn(g, B, L, hid, dtype=torch.bfloat16).to(DEV)
+    y = randn(g, B, L, hid, dtype=torch.bfloat16).to(DEV)
+    mod = randn(g, B, 1, 3 * hid, dtype=torch.bfloat16).to(DEV)
+    gate = mod.chunk(3, dim=-1)[2]                              # a strided [B, 1, hid] chunk of the modulation vector
+    out = _gated_residual(x, gate, y)
+    assert torch.equal(out, oracle.gated_residual_ref(x, gate, y))
+    # and it differs from the single-rounding form somewhere, i.e. the flag does something
+    if B * L * hid > 10000:
+        once = (x.float() + gate.float() * y.float()).to(torch.bfloat16)
+        assert not torch.equal(out, once)

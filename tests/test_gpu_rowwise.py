@@ -4,6 +4,8 @@ The fp32 grids mirror the reference's own unit tests (tests/test_rms_norm.py, te
 test_rope.py: fp32, atol 1e-5 forward, 1e-3 backward); the bf16 cases use the tolerance stated for
 this path (atol 1e-2, rtol 1e-2) at the Flux shapes, plus ragged and strided edge cases.
 """
+import math
+
 import pytest
 import torch
 
@@ -45,6 +47,40 @@ def test_rms_norm_bf16_shapes(shape):
     # scale kept in fp32 (a module that was not cast): output stays bf16 as in the reference launcher
     y2 = tk.rms_norm(x, w.float())
     torch.testing.assert_close(y2, oracle.rms_norm_ref(x, w.float()).to(torch.bfloat16), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 24, 4608, 128),   # the Flux q/k shape: one vector per lane
+                                   (3, 700, 512),         # two vectors per lane
+                                   (2, 333, 1536),        # three
+                                   (2, 100, 2048),        # four
+                                   (2, 37, 4104),         # more than four: one block per row
+                                   (1, 19, 10000),
+                                   (5, 9, 100),           # not a multiple of the vector width: one block per row
+                                   (4, 64)])
+def test_rms_norm_bf16_backward(shape, scale_dtype):
+    """_rms_norm.backward (kernels/normalization.py:110-139) for bf16 activations, with the scale in bf16
+    or kept in fp32, over every register plan of the backward kernel and its one-block-per-row
+    fallback. dx against autograd of the oracle at bf16 tolerance; dscale, an fp32 sum over all rows,
+    against the same sum formed in fp64 from the oracle's per-row terms."""
+    g = seeded(sum(shape) + (scale_dtype == torch.float32))
+    x = randn(g, *shape, dtype=torch.bfloat16).to(DEV).requires_grad_(True)
+    w = (torch.rand(shape[-1], generator=g) + 0.5).to(scale_dtype).to(DEV).requires_grad_(True)
+    dy = randn(g, *shape, dtype=torch.bfloat16).to(DEV)
+    y = tk.rms_norm(x, w)
+    y.backward(dy)
+    assert x.grad.dtype == torch.bfloat16 and w.grad.dtype == scale_dtype and w.grad.shape == w.shape
+    # fp32 oracle of the same function (bf16 values, fp32 arithmetic, no intermediate rounding)
+    dx_ref, dw_ref = oracle.rms_norm_bwd_ref(x.detach().float(), w.detach().float(), dy.float())
+    torch.testing.assert_close(x.grad.float(), dx_ref, atol=1e-2 * max(1.0, dx_ref.abs().max().item()), rtol=1e-2)
+    assert (x.grad.float() - dx_ref).abs().mean().item() < 4e-3
+    # dscale[c] = sum_rows dy * x * rstd: a sum of rows terms of size ~1, so its error scales with sqrt(rows)
+    xf = x.detach().double()
+    rstd = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)
+    dw64 = (dy.double() * xf * rstd).reshape(-1, shape[-1]).sum(0)
+    torch.testing.assert_close(dw_ref.double(), dw64, atol=1e-3 * math.sqrt(xf.numel() / shape[-1]), rtol=1e-3)  # the oracle agrees with the closed form
+    tol = (2.0 ** -8 if scale_dtype == torch.bfloat16 else 1e-5) * dw64.abs() + 2e-4 * math.sqrt(xf.numel() / shape[-1])
+    assert ((w.grad.double() - dw64).abs() <= tol).all()
 
 
 def test_rms_norm_config1_cpu_oracle_and_strided_view():
@@ -144,6 +180,31 @@ def test_config3_rope_concat_bit_exact_parts():
     torch.testing.assert_close(q2, rq, atol=1e-2, rtol=1e-2)
     torch.testing.assert_close(k2, rk, atol=1e-2, rtol=1e-2)
     assert torch.equal(v2, torch.cat((txt[2], img[2]), 2))
+
+
+def test_config3_whole_at_full_size():
+    """RoPE with the EmbedND table plus the txt/img concat at the full 512 + 64 x 64 positions, 24 heads:
+    one fused launch against the oracle chain (torch.cat along the sequence, then apply_rope), v
+    bit-exact, q and k at the bf16 tolerance and at one rounding of the fp32 value; the same through
+    the two separate operators (concat, then apply_rope)."""
+    txt, img, pe = cfg.config3(DEV)
+    assert txt[0].shape == (1, 24, 512, 128) and img[0].shape == (1, 24, 4096, 128) and pe.shape == (1, 1, 4608, 64, 2, 2)
+    cat = [torch.cat((t, i), dim=2) for t, i in zip(txt, img)]
+    rq, rk = oracle.apply_rope_ref(cat[0], cat[1], pe)
+    q, k, v = tk.qkv_prep(img[0], img[1], img[2], txt[0], txt[1], txt[2], pe=pe)
+    assert torch.equal(v, cat[2])
+    for got, want, src in ((q, rq, cat[0]), (k, rk, cat[1])):
+        torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+        # the rotation in fp32 from the bf16 inputs, rounded once
+        x_ = src.float().reshape(*src.shape[:-1], -1, 1, 2)
+        w32 = (pe[..., 0] * x_[..., 0] + pe[..., 1] * x_[..., 1]).reshape(src.shape)
+        assert ((got.float() - w32).abs() <= w32.abs() * 2.0 ** -8 * 1.01 + 1e-6).all()
+    # rotations preserve the norm of every (even, odd) pair: |q_rot| == |q| row by row up to rounding
+    torch.testing.assert_close(q.float().pow(2).sum(-1), cat[0].float().pow(2).sum(-1), rtol=5e-3, atol=0)
+    q0, k0, v0 = tk.qkv_prep(img[0], img[1], img[2], txt[0], txt[1], txt[2])
+    assert all(torch.equal(a, b) for a, b in zip((q0, k0, v0), cat))
+    q1, k1 = tk.apply_rope(q0, k0, pe)
+    assert torch.equal(q1, q) and torch.equal(k1, k)
 
 
 def test_qkv_prep_norm_rope_matches_unfused_sequence():

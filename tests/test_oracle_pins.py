@@ -263,3 +263,53 @@ def test_single_block_oracle_equals_unfused_composition():
     a = oracle.attention_ref_fp32(q, k, v).permute(0, 2, 1, 3).reshape(1, L, hid)
     out = oracle.linear_ref(torch.cat((a, oracle.gelu_tanh_ref(y1[..., 3 * hid:])), 2), sd["linear2.weight"], sd["linear2.bias"])
     torch.testing.assert_close(got, oracle.gated_residual_ref(x, gate, out), rtol=1e-5, atol=1e-5)
+
+
+def test_double_block_oracle_equals_unfused_composition():
+    """The double-stream oracle (modules/blocks.py:126-171) is the pinned per-op oracles chained in the
+    reference's order: per stream mod1 -> qkv -> QKNorm, txt-first concat, RoPE, attention, then per
+    stream proj + gated residual, mod2 -> mlp (GELU) -> gated residual."""
+    g = rng(12)
+    hid, heads, Li, Lt = 32, 2, 7, 3
+    mlp = 4 * hid
+    D = hid // heads
+    sd = {}
+    for s_ in ("img", "txt"):
+        sd[f"{s_}_mod.lin.weight"] = torch.randn(6 * hid, hid, generator=g) * 0.2
+        sd[f"{s_}_mod.lin.bias"] = torch.randn(6 * hid, generator=g) * 0.1
+        sd[f"{s_}_attn.qkv.weight"] = torch.randn(3 * hid, hid, generator=g) * 0.2
+        sd[f"{s_}_attn.qkv.bias"] = torch.randn(3 * hid, generator=g) * 0.1
+        sd[f"{s_}_attn.norm.query_norm.scale"] = torch.rand(D, generator=g) + 0.5
+        sd[f"{s_}_attn.norm.key_norm.scale"] = torch.rand(D, generator=g) + 0.5
+        sd[f"{s_}_attn.proj.weight"] = torch.randn(hid, hid, generator=g) * 0.2
+        sd[f"{s_}_attn.proj.bias"] = torch.randn(hid, generator=g) * 0.1
+        sd[f"{s_}_mlp.0.weight"] = torch.randn(mlp, hid, generator=g) * 0.2
+        sd[f"{s_}_mlp.0.bias"] = torch.randn(mlp, generator=g) * 0.1
+        sd[f"{s_}_mlp.2.weight"] = torch.randn(hid, mlp, generator=g) * 0.1
+        sd[f"{s_}_mlp.2.bias"] = torch.randn(hid, generator=g) * 0.1
+    B = 2
+    xs = {"img": torch.randn(B, Li, hid, generator=g), "txt": torch.randn(B, Lt, hid, generator=g)}
+    vec = torch.randn(B, hid, generator=g)
+    pe = torch.randn(1, 1, Lt + Li, D // 2, 2, 2, generator=g)
+    g_img, g_txt = oracle.double_stream_block_ref(sd, xs["img"], xs["txt"], vec, pe, heads)
+
+    mods, qkv = {}, {}
+    for s_ in ("img", "txt"):
+        mods[s_] = oracle.linear_ref(oracle.silu_ref(vec), sd[f"{s_}_mod.lin.weight"], sd[f"{s_}_mod.lin.bias"])[:, None].chunk(6, -1)
+        xm = oracle.layer_norm_modulation_ref(xs[s_], mods[s_][1], mods[s_][0], eps=1e-6)
+        # the same through the reference's inductor-derived op (ops/modulation.py:5-27, mod1) on the normalised rows
+        ln = F.layer_norm(xs[s_], (hid,), eps=1e-6)
+        torch.testing.assert_close(oracle.modulation_scale_shift_ref(ln, torch.cat(mods[s_], -1)[:, 0], True), xm, rtol=1e-5, atol=1e-5)
+        q, k, v = oracle.split_heads_ref(oracle.linear_ref(xm, sd[f"{s_}_attn.qkv.weight"], sd[f"{s_}_attn.qkv.bias"]), heads)
+        qkv[s_] = (oracle.rms_norm_ref(q, sd[f"{s_}_attn.norm.query_norm.scale"]), oracle.rms_norm_ref(k, sd[f"{s_}_attn.norm.key_norm.scale"]), v)
+    q, k, v = (torch.cat((qkv["txt"][i], qkv["img"][i]), dim=2) for i in range(3))
+    q, k = oracle.apply_rope_ref(q, k, pe)
+    attn = oracle.attention_ref_fp32(q, k, v).permute(0, 2, 1, 3).reshape(B, Lt + Li, hid)
+    parts = {"txt": attn[:, :Lt], "img": attn[:, Lt:]}
+    for s_, got in (("img", g_img), ("txt", g_txt)):
+        shift1, scale1, gate1, shift2, scale2, gate2 = mods[s_]
+        x = oracle.gated_residual_ref(xs[s_], gate1, oracle.linear_ref(parts[s_], sd[f"{s_}_attn.proj.weight"], sd[f"{s_}_attn.proj.bias"]))
+        xm = oracle.layer_norm_modulation_ref(x, scale2, shift2, eps=1e-6)
+        h = oracle.linear_ref(xm, sd[f"{s_}_mlp.0.weight"], sd[f"{s_}_mlp.0.bias"], "GELU")
+        want = oracle.gated_residual_ref(x, gate2, oracle.linear_ref(h, sd[f"{s_}_mlp.2.weight"], sd[f"{s_}_mlp.2.bias"]))
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)

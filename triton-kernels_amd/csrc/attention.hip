@@ -28,6 +28,7 @@
 // read): at that point K(t+1) is retired and refilled with K(t+3), while the V buffer being
 // refilled is the one read a whole iteration earlier.
 #include "common.h"
+#include "attention_params.h"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -38,17 +39,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-struct AttnParams {
-    const bf16_t* q; const bf16_t* k; const bf16_t* v; bf16_t* o; float* lse;
-    int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, o_sb, o_sh, o_sl;
-    int H, L, n_qtiles, total_tiles;
-    float scale_log2;  // sm_scale * log2(e)
-    // 64-row-per-wave kernel only: query rows of a launch. (batch*head) pairs are taken two at a
-    // time; the even one gets cnt_even tiles starting at row first_even, the odd one cnt_odd tiles
-    // from first_odd.
-    int cnt_even, cnt_odd, first_even, first_odd;
-};
 
 constexpr unsigned kAttnRsrcFlags = 0x00020000u;
 
@@ -467,20 +457,29 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
 // buffers and two P^T buffers need more than 256, so one wave per SIMD runs and the instruction
 // stream itself has to keep the matrix pipe fed, the way a GEMM main loop does.
 //
-//   * Work is cut into sub-tiles of 32 keys. Iteration u issues 64 MFMAs: 32 for S^T(u+1) =
-//     K(u+1) Q^T and 32 for O^T += V(u-1)^T P(u-1)^T, while the VALU turns S^T(u) into P^T(u), one
-//     VALU instruction behind each MFMA. LDS fragment reads are issued eight slots ahead of use.
+//   * Work is cut into sub-tiles of 32 keys. Iteration u issues 16*QB MFMAs (QB = 16-row query
+//     blocks per wave, 64 MFMAs for QB = 4): half of them for S^T(u+1) = K(u+1) Q^T, half for
+//     O^T += V(u-1)^T P(u-1)^T, while the VALU turns S^T(u) into P^T(u) in the gaps between them:
+//     a constexpr schedule (attn_sched) gives every MFMA slot either one exponential or up to two
+//     other steps (convert, sums), because a single wave issues one instruction per four cycles
+//     and an exponential takes two such issue slots. LDS fragment reads run 3*QB slots ahead.
 //   * Q is scaled by sm_scale*log2(e) and rounded to bf16 once; the first MFMA of every S^T
 //     accumulator takes "-m" (the row's reference maximum, one register block per 16 rows) as its
 //     C operand, so exp2 applies to the MFMA result directly: no multiply, no subtract.
-//   * The reference maximum is not the running maximum: it is only moved when a row's partial sum
-//     of a sub-tile exceeds 2^40 (which also catches inf). exp2(s - m) is then simply larger than
-//     one for a while, which costs no accuracy in fp32 / bf16 (relative precision), and the common
-//     path has no max, no compare per element and no rescale. When the test fires (first sub-tile
-//     aside this needs scores to grow by more than 40 in the log2 domain) the whole wave
-//     re-bases: true row maxima, accumulators, sums and the S^T blocks in flight are shifted.
-//   * K and V tiles of 64 keys go through two LDS rings of four (128 KB) so that every LDS offset
-//     in the four-tile body is a compile-time constant; one workgroup barrier per 64 keys.
+//   * The reference maximum is not the running maximum: it is only moved when a lane's partial sum
+//     of a sub-tile reaches 2^40 (which also catches inf and NaN). exp2(s - m) is then simply
+//     larger than one for a while, which costs no accuracy in fp32 / bf16 (relative precision),
+//     and the common path has no max, no compare per element and no rescale. When the test fires
+//     (first sub-tile aside this needs scores to grow by more than 40 in the log2 domain) the
+//     whole wave re-bases: true row maxima, accumulators, sums and the S^T blocks in flight are
+//     shifted. Row sums are fp32 sums of the unrounded exponentials.
+//   * K and V tiles of 64 keys go through two LDS rings of four 16 KB buffers (128 KB). The loop
+//     body is unrolled over the four ring positions, so every LDS offset is a compile-time
+//     constant; one workgroup barrier per 64 keys, with this wave's own loads of the tile about
+//     to be read waited for in front of it. Tiles are fetched with LDS-writing buffer loads
+//     through running descriptors (base advanced per tile, rows past the end read as zero).
+//   * The ragged tail (keys past L in the last tile) is handled by a second copy of the body that
+//     adds a -inf mask to the seed; the common loop carries no such test.
 // ------------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -488,8 +487,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // Left to the compiler, a kernel with more than 256 registers gets accumulation-register MFMAs for
 // everything and a copy in front of every VALU use, or keeps the "a"-constrained operands in vector
 // registers and copies them over in front of every MFMA.
-//   * The accumulation registers are addressed by number: a[0:127] = O^T accumulators, block
-//     (db, qb) at a[16*db + 4*qb ..+3]; a[128:191] = Q fragments, (qb, ks) at a[128 + 16*qb + 4*ks ..+3].
+//   * The accumulation registers are addressed by number: a[0 : 32*QB-1] = O^T accumulators, block
+//     (db, qb) at a[4*(db*QB + qb) ..+3]; the next 16*QB hold the Q fragments, (qb, ks) at
+//     a[32*QB + 16*qb + 4*ks ..+3].
 //     The compiler never sees them (attn_claim_agprs only makes the kernel descriptor reserve
 //     them), so it must not use accumulation registers of its own: the kernel has to fit the 256
 //     vector registers without spilling, which tests/test_abi.py checks on the generated code.
@@ -651,7 +651,7 @@ constexpr int attn_load_slot(int j, int ns, int bs, int sp, bool second) {
 }
 
 // QB = 16-row query blocks per wave, NW = waves per workgroup: 16*QB*NW query rows per workgroup.
-//   <4, 4>: 64 rows per wave, 256 per workgroup, one wave per SIMD (428 registers).
+//   <4, 4>: 64 rows per wave, 256 per workgroup, one wave per SIMD (248 vector + 192 accumulation registers).
 //   <3, 4>: 48 rows per wave, 192 per workgroup: the same code with three quarters of the work per
 //           iteration, for the launch that evens out the last round (see attn_launch_w64).
 template <int QB, int NW>
@@ -1143,7 +1143,8 @@ static bool view_ok(const void* ptr, int64_t sb, int64_t sh, int64_t sl) {
 extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     if (!a) return fail(FLUX_E_NULL, "flux_attention_fwd_bf16: null args");
     if (a->B < 0 || a->H <= 0 || a->L < 0) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: bad shape B=%lld H=%lld L=%lld", (long long)a->B, (long long)a->H, (long long)a->L);
-    if (a->D != 64 && a->D != 128) return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: head dim %d not supported (64, 128)", a->D);
+    if (a->D != 16 && a->D != 32 && a->D != 64 && a->D != 128 && a->D != 256)
+        return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: head dim %d not supported (16, 32, 64, 128, 256)", a->D);
     if (!(a->sm_scale == a->sm_scale)) return fail(FLUX_E_UNSUPPORTED, "flux_attention_fwd_bf16: sm_scale is NaN");
     if (a->B == 0 || a->L == 0) return FLUX_OK;
     if (a->L > 0x7fffffff / 64 || a->B * a->H > 0x7fffffff / 64) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: problem too large");
@@ -1166,7 +1167,10 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     // Head dim 128: 64 rows per wave (256 per workgroup, one workgroup per CU) once there are enough
     // such tiles to occupy the chip; smaller problems get 128-row workgroups, two per CU.
     const int64_t tiles256 = BH * ((a->L + 255) / 256);
-    if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64(p, BH, st);
+    if (a->D != 64 && a->D != 128) {
+        if (BH * ((a->L + 63) / 64) > 0x7fffffffLL) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: problem too large");
+        attn_launch_plain(p, BH, a->D, st);
+    } else if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64(p, BH, st);
     else if (a->D == 128) attn_launch_pipe<128, 1, 64>(p, BH, st);
     else attn_launch_pipe<64, 1, 64>(p, BH, st);
     return check_launch("flux_attention_fwd_bf16");

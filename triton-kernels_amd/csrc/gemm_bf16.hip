@@ -836,16 +836,6 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
-// FLUX_GEMM_TILE=256, 128 or 64 forces the tile size (for measurements); anything else = automatic.
-static int forced_tile() {
-    static int v = [] {
-        const char* e = getenv("FLUX_GEMM_TILE");
-        const int t = e ? atoi(e) : 0;
-        return (t == 256 || t == 128 || t == 64) ? t : 0;
-    }();
-    return v;
-}
-
 }  // namespace flux
 
 using namespace flux;
@@ -936,12 +926,11 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     // per CU) spread the work better than they lose in operand re-reads.
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
     const int64_t mid_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
-    const int tile = forced_tile();
     // 256-wide tiles once they fill most of the chip; below that 128-wide ones (two workgroups per
     // CU); problems with too few of those to give every second CU one are bound by the latency of
     // the K loop and run on 64-wide tiles, four times as many workgroups.
-    if (tile == 256 || (tile == 0 && big_tiles >= 160)) launch_tiled<4>(p, st);
-    else if (tile == 64 || (tile == 0 && mid_tiles <= 64)) launch_tiled<1>(p, st);
+    if (big_tiles >= 160) launch_tiled<4>(p, st);
+    else if (mid_tiles <= 64) launch_tiled<1>(p, st);
     else launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
 }

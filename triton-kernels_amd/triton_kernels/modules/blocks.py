@@ -247,15 +247,21 @@ class DoubleStreamBlock(nn.Module):
     # leave most CUs idle when they run alone, so the fused path runs the txt chain on a second HIP
     # stream of default priority, next to the img chain, and joins the two around the joint attention.
     two_streams = True
-    _side_streams: dict = {}
 
-    @classmethod
-    def _side_stream(cls, dev: torch.device) -> "torch.cuda.Stream":
-        st = cls._side_streams.get(dev.index)
+    def _side_stream(self, dev: torch.device) -> "torch.cuda.Stream":
+        """This block's second stream on `dev`. Each instance keeps its own (per device), so two blocks
+        driven from different host threads or streams never order their txt chains behind each
+        other; setdefault makes the lazy creation safe when one instance is called from two threads."""
+        streams = self.__dict__.setdefault("_side_streams", {})
+        st = streams.get(dev.index)
         if st is None:
-            st = torch.cuda.Stream(device=dev)
-            cls._side_streams[dev.index] = st
+            st = streams.setdefault(dev.index, torch.cuda.Stream(device=dev))
         return st
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state.pop("_side_streams", None)   # streams are neither copied nor pickled with the block
+        return state
 
     def forward(self, img: Tensor, txt: Tensor, vec: Tensor, pe: Tensor) -> tuple[Tensor, Tensor]:
         H = self.num_heads
