@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FLUX_ABI_VERSION 2
+#define FLUX_ABI_VERSION 3
 
 enum flux_dtype { FLUX_BF16 = 0, FLUX_F32 = 1 };
 
@@ -38,7 +38,7 @@ enum flux_status {
     FLUX_E_UNSUPPORTED = -6
 };
 
-enum flux_activation { FLUX_ACT_NONE = 0, FLUX_ACT_GELU_TANH = 1 };
+enum flux_activation { FLUX_ACT_NONE = 0, FLUX_ACT_GELU_TANH = 1, FLUX_ACT_SILU = 2 };
 
 /* Largest row a row-wise kernel accepts; mirrors MAX_FUSED_SIZE in kernels/utils.py:6-11. */
 #define FLUX_MAX_ROW 65536
@@ -123,6 +123,9 @@ int flux_qkv_prep(const flux_qkv_prep_args* args, void* stream);
  * Replaces linear / _linear_fwd / gelu (kernels/linear.py:104-151, 31-101, 22-28) and the raw
  * triton_linear (ops/linear.py:5-71).
  * A is [M,K] with row stride lda, W is [N,K] (nn.Linear layout) with row stride ldw.
+ * in_act == FLUX_ACT_SILU applies x * sigmoid(x) (fp32, rounded to bf16, as flux_silu does) to A on
+ * the way in: lin(silu(vec)) of Modulation (modules/blocks.py:62-67) as one launch. Only for
+ * M <= 8 (the row-vector path); larger M returns FLUX_E_UNSUPPORTED.
  *
  * Epilogue, applied in this order on the fp32 accumulator:
  *   + bias[n] (nullable)
@@ -164,7 +167,7 @@ typedef struct flux_linear_args {
     int64_t lda, ldw, ldy, ldy2;
     int64_t split_n, y2_col0;
     int64_t ldresid, gate_batch_stride, rows_per_batch;
-    int32_t act; int64_t act_begin;
+    int32_t act; int32_t in_act; int64_t act_begin;
     const flux_linear_qk_fusion* qk;           /* null = off */
 } flux_linear_args;
 

@@ -174,3 +174,42 @@ def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
     rq, rk = oracle.apply_rope_ref(qn, kn, pe.cpu())
     torch.testing.assert_close(q.cpu(), rq, atol=2e-2, rtol=2e-2)
     torch.testing.assert_close(k.cpu(), rk, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("M", [1, 2, 5, 8])
+@pytest.mark.parametrize("N,K", [(9216, 3072), (18432, 3072), (40, 72), (33, 50)])
+def test_linear_input_silu_is_modulation(M, N, K):
+    """lin(silu(vec)) of Modulation (modules/blocks.py:62-67) as one launch: SiLU in fp32 rounded to bf16
+    on the way in, bit-identical to the two-launch form and within tolerance of the oracle."""
+    from triton_kernels.modules.blocks import _silu
+    g = seeded(M + N + K)
+    vec = randn(g, M, K, dtype=torch.bfloat16, std=2.0).to(DEV)
+    w = randn(g, N, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16, std=0.02).to(DEV)
+    fused = tk.linear_into(vec, w, b, in_activation="SiLU")
+    two = tk.linear(_silu(vec), w, b)
+    assert torch.equal(fused, two)
+    ref32 = oracle.linear_ref_fp32(oracle.silu_ref(vec), w, b)
+    torch.testing.assert_close(fused.float(), ref32, atol=2e-2, rtol=1e-2)
+
+
+def test_linear_input_silu_needs_few_rows_and_modulation_uses_it():
+    g = seeded(3)
+    vec = randn(g, 9, 64, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, 32, 64, dtype=torch.bfloat16).to(DEV)
+    with pytest.raises(AssertionError):
+        tk.linear_into(vec, w, None, in_activation="SiLU")
+    from triton_kernels.modules.blocks import Modulation
+    torch.manual_seed(0)
+    mod = Modulation(256, double=True).to(torch.bfloat16).to(DEV)
+    for rows in (1, 3, 9):                                    # 9 rows: the two-launch form
+        v = randn(g, rows, 256, dtype=torch.bfloat16).to(DEV)
+        m1, m2 = mod(v)
+        want = oracle.linear_ref_fp32(oracle.silu_ref(v), mod.lin.weight, mod.lin.bias)[:, None, :].chunk(6, dim=-1)
+        for got, ref in zip((m1.shift, m1.scale, m1.gate, m2.shift, m2.scale, m2.gate), want):
+            assert got.shape == (rows, 1, 256)
+            torch.testing.assert_close(got.float(), ref, atol=2e-2, rtol=1e-2)
+        mod.fused_silu = False
+        u1, _ = mod(v)
+        mod.fused_silu = True
+        assert torch.equal(u1.scale, m1.scale)

@@ -169,6 +169,22 @@ def test_rope_bf16_flux_table_and_per_batch_pe():
     torch.testing.assert_close(ok, rk, atol=1e-2, rtol=1e-2)
 
 
+def test_rope_table_with_a_head_extent_uses_the_first_head():
+    """kernels/positional_embedding.py:31-32 indexes the table by position only, so a [1, H, L, D/2, 2, 2]
+    table behaves like its first head's."""
+    g = seeded(33)
+    B, H, L, D = 2, 3, 40, 64
+    q = randn(g, B, H, L, D, dtype=torch.bfloat16).to(DEV)
+    k = randn(g, B, H, L, D, dtype=torch.bfloat16).to(DEV)
+    pe = randn(g, 1, H, L, D // 2, 2, 2).to(DEV)
+    q1, k1 = tk.apply_rope(q, k, pe)
+    q0, k0 = tk.apply_rope(q, k, pe[:, :1])
+    assert torch.equal(q1, q0) and torch.equal(k1, k0)
+    rq, rk = oracle.apply_rope_ref(q, k, pe[:, :1])
+    torch.testing.assert_close(q1, rq, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(k1, rk, atol=1e-2, rtol=1e-2)
+
+
 def test_config3_rope_concat_bit_exact_parts():
     """txt/img concat along the sequence is bit-exact; q,k are rotated on the way, v is copied."""
     txt, img, pe = cfg.config3(DEV, n_txt=64, grid=16)

@@ -37,6 +37,7 @@ struct GemmParams {
     int64_t lda, ldw, ldy, ldy2, ldresid, gate_stride;
     int split_n, y2_col0, rows_per_batch;
     int act, act_begin;
+    int in_silu;  // 1: A passes through x * sigmoid(x), rounded to bf16, on the way in (row-vector and scalar kernels)
     int tiles_m, tiles_n, group_m;
     int bias_vec;  // 1: bias may be read with 8-byte buffer loads (4-byte aligned base)
     int vec_io;  // 1: every output/residual row segment of 8 columns may be accessed as 16 bytes
@@ -609,7 +610,9 @@ __device__ __forceinline__ void gemm_tile_slabs(const GemmParams& p, char* lds, 
         else xa[buf][r - FN] = *reinterpret_cast<const bf16x8*>(pa + (r - FN) * 16 * ROWB);
     };
     auto mfma_one = [&](int buf, int idx) {
-        const int i = idx / FN, j = idx % FN;
+        // boustrophedon over the accumulator grid: from one MFMA to the next only one of the two
+        // operands changes, also at the end of a row (about 1 % less time at the power limit)
+        const int i = idx / FN, j = (i & 1) ? FN - 1 - idx % FN : idx % FN;
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
     };
 
@@ -754,6 +757,10 @@ __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
                 const Vec16<bf16_t> a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) af[m][e] = bf2f(a.v[e]);
+                if (p.in_silu) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) af[m][e] = bf2f(f2bf(af[m][e] * __builtin_amdgcn_rcpf(1.0f + __expf(-af[m][e]))));
+                }
             }
 #pragma unroll
             for (int c = 0; c < CPW; ++c)
@@ -810,7 +817,11 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     const bf16_t* a = p.A + static_cast<int64_t>(m) * p.lda;
     const bf16_t* w = p.W + static_cast<int64_t>(n) * p.ldw;
     float acc = 0.0f;
-    for (int k = 0; k < p.K; ++k) acc += bf2f(a[k]) * bf2f(w[k]);
+    for (int k = 0; k < p.K; ++k) {
+        float x = bf2f(a[k]);
+        if (p.in_silu) x = bf2f(f2bf(x * __builtin_amdgcn_rcpf(1.0f + __expf(-x))));
+        acc += x * bf2f(w[k]);
+    }
     float t = acc + (p.bias ? bf2f(p.bias[n]) : 0.0f);
     if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
     t = bf2f(f2bf(t));
@@ -848,6 +859,8 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     if (a->M == 0 || a->N == 0) return FLUX_OK;
     if (a->lda < a->K || a->ldw < a->K) return fail(FLUX_E_SHAPE, "flux_linear_bf16: leading dimension smaller than K");
     if (a->act != FLUX_ACT_NONE && a->act != FLUX_ACT_GELU_TANH) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: unknown activation %d", a->act);
+    if (a->in_act != FLUX_ACT_NONE && a->in_act != FLUX_ACT_SILU) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: unknown input activation %d", a->in_act);
+    if (a->in_act == FLUX_ACT_SILU && (a->M > 8 || a->qk != nullptr)) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: input SiLU is for M <= 8 without the qk fusion (M=%lld)", (long long)a->M);
     const bool split = a->Y2 != nullptr && a->split_n < a->N;
     if (split && (a->split_n < 0 || a->y2_col0 < 0)) return fail(FLUX_E_SHAPE, "flux_linear_bf16: bad split");
     if ((a->gate == nullptr) != (a->resid == nullptr)) return fail(FLUX_E_NULL, "flux_linear_bf16: gate and resid go together");
@@ -863,6 +876,7 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     p.split_n = split ? (int)a->split_n : p.N;
     p.y2_col0 = split ? (int)a->y2_col0 : 0;
     p.rows_per_batch = a->gate ? (int)a->rows_per_batch : 1;
+    p.in_silu = a->in_act == FLUX_ACT_SILU;
     p.act = a->act; p.act_begin = (int)(a->act_begin < 0 ? 0 : (a->act_begin > a->N ? a->N : a->act_begin));
     p.tiles_m = p.tiles_n = 0; p.group_m = 4;
     p.bias_vec = a->bias != nullptr && (reinterpret_cast<uintptr_t>(a->bias) & 3u) == 0 && a->N % 4 == 0;

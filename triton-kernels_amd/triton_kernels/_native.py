@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfluxhip
 _lib = None
 
 FLUX_BF16, FLUX_F32 = 0, 1
-ACT_NONE, ACT_GELU_TANH = 0, 1
+ACT_NONE, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
 E_NULL, E_SHAPE, E_DTYPE, E_ALIGN, E_TOO_WIDE, E_UNSUPPORTED = -1, -2, -3, -4, -5, -6
 MAX_ROW = 65536
 
@@ -59,7 +59,7 @@ class LinearArgs(Structure):
         ("lda", c_int64), ("ldw", c_int64), ("ldy", c_int64), ("ldy2", c_int64),
         ("split_n", c_int64), ("y2_col0", c_int64),
         ("ldresid", c_int64), ("gate_batch_stride", c_int64), ("rows_per_batch", c_int64),
-        ("act", c_int32), ("act_begin", c_int64),
+        ("act", c_int32), ("in_act", c_int32), ("act_begin", c_int64),
         ("qk", POINTER(LinearQKFusion)),
     ]
 
@@ -116,7 +116,7 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.flux_abi_version() != 2:
+        if handle.flux_abi_version() != 3:
             raise RuntimeError("libfluxhip.so: ABI version mismatch")
         _lib = handle
     return _lib
@@ -204,5 +204,5 @@ def src4(t: torch.Tensor | None) -> Src4:
 __all__ = [
     "lib", "lib_path", "check", "last_error", "dtype_code", "require_gpu", "stream_ptr", "on_device", "ptr", "src4",
     "Src4", "QkvPrepArgs", "LinearArgs", "AttnArgs", "SIGNATURES", "byref",
-    "FLUX_BF16", "FLUX_F32", "ACT_NONE", "ACT_GELU_TANH", "MAX_ROW",
+    "FLUX_BF16", "FLUX_F32", "ACT_NONE", "ACT_GELU_TANH", "ACT_SILU", "MAX_ROW",
 ]

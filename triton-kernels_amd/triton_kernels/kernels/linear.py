@@ -25,13 +25,15 @@ def _rows_2d(x: Tensor, K: int) -> Tensor:
 
 def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "", act_begin: int = 0,
                 out: Tensor | None = None, out2: Tensor | None = None, split: int | None = None,
-                resid: Tensor | None = None, gate: Tensor | None = None, qk: dict | None = None) -> Tensor:
+                resid: Tensor | None = None, gate: Tensor | None = None, qk: dict | None = None,
+                in_activation: str = "") -> Tensor:
     """General form of the fused linear.
 
     out   : [M, >=split] destination (row stride free) for columns [0, split)
     out2  : destination for columns [split, N), written starting at its column 0
     act_begin : GELU applies to columns >= act_begin only
     resid, gate : y = resid + gate * y with resid [..., N] and gate [B, 1, N] (or [B, N])
+    in_activation : "SiLU" applies x * sigmoid(x) (rounded to bf16) to x on the way in; at most 8 rows
     qk    : QK RMSNorm + RoPE on the way out for the leading 2 * heads * 128 columns (q heads, then k
             heads), which then go to q_out / k_out [B, heads, out_len, 128] instead of `out`:
             dict(q_out, k_out, q_scale, k_scale, pe, heads, seq_len, pos0=0, eps=1e-6); see
@@ -80,6 +82,8 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
         a.resid, a.ldresid = r2.data_ptr(), r2.stride(0)
         a.gate, a.gate_batch_stride, a.rows_per_batch = g2.data_ptr(), (g2.stride(0) if nb > 1 else N), M // nb
     a.act, a.act_begin = act, act_begin
+    a.in_act = {"": nv.ACT_NONE, "SiLU": nv.ACT_SILU}[in_activation]
+    assert a.in_act == nv.ACT_NONE or M <= 8, "the input activation is fused for at most 8 rows"
     keep = None
     if qk is not None:
         f = nv.LinearQKFusion()

@@ -18,8 +18,13 @@ def _row_view(t: Tensor) -> Tensor:
 
 def _pe_table(pe: Tensor, B: int, L: int, D: int) -> tuple[Tensor, int]:
     """fp32 [.., L, D/2, 2, 2] -> contiguous table and its batch stride (0 = shared by all batches).
-    A head extent other than 1 is not supported (the reference kernel ignores it altogether)."""
+    The reference kernel reads the first [L, D/2, 2, 2] table whatever the leading extents are
+    (kernels/positional_embedding.py:31-32). A head extent is treated the same way here (the first
+    head's table serves all heads); a batch extent equal to B is honoured, as broadcasting in the
+    plain-PyTorch apply_rope would."""
     assert pe.shape[-4:] == (L, D // 2, 2, 2), f"freqs_cis must end in [{L}, {D // 2}, 2, 2], got {tuple(pe.shape)}"
+    if pe.dim() >= 6 and pe.shape[-5] > 1:
+        pe = pe.narrow(-5, 0, 1)
     lead = pe.shape[:-4]
     if pe.dtype != torch.float32:
         pe = pe.float()

@@ -123,6 +123,8 @@ class ModulationOut:
 
 
 class Modulation(nn.Module):
+    fused_silu = True
+
     def __init__(self, dim: int, double: bool):
         super().__init__()
         self.is_double = double
@@ -130,7 +132,13 @@ class Modulation(nn.Module):
         self.lin = Linear(dim, self.multiplier * dim, bias=True)
 
     def forward(self, vec: Tensor) -> tuple[ModulationOut, ModulationOut | None]:
-        chunks = self.lin(_silu(vec))[:, None, :].chunk(self.multiplier, dim=-1)
+        rows = vec.numel() // vec.shape[-1]
+        if self.fused_silu and vec.is_cuda and vec.dtype == torch.bfloat16 and rows <= 8:
+            # one launch: the row-vector kernel applies SiLU to vec as it reads it
+            out = linear_into(vec, self.lin.weight, self.lin.bias, in_activation="SiLU").reshape(*vec.shape[:-1], -1)
+        else:
+            out = self.lin(_silu(vec))
+        chunks = out[:, None, :].chunk(self.multiplier, dim=-1)
         first = ModulationOut(*chunks[:3])
         return first, (ModulationOut(*chunks[3:]) if self.is_double else None)
 
