@@ -213,3 +213,29 @@ def test_linear_input_silu_needs_few_rows_and_modulation_uses_it():
         u1, _ = mod(v)
         mod.fused_silu = True
         assert torch.equal(u1.scale, m1.scale)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_linear_head_and_tail_launches(gated):
+    """4608 x 12288 outputs are 864 tiles of 256 x 256, 3.375 rounds of 256 CUs: the library launches the
+    first 4096 rows on those tiles and the last 512 rows on 128-wide ones. Same results as one launch
+    would give: compared with the fp32 product row block by row block."""
+    g = seeded(77 + gated)
+    M, N, K = 4608, 12288, 192
+    a = randn(g, M, K, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, N, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16, std=0.02).to(DEV)
+    if not gated:
+        y = tk.linear(a, w, b, activation="GELU")
+        ref32 = oracle.linear_ref_fp32(a, w, b, "GELU")
+        assert ((y.float() - ref32).abs() <= half_ulp_bound(ref32)).all()
+        return
+    B, L = 9, 512                                               # the cut at row 4096 falls between batch elements
+    x = randn(g, B, L, N, dtype=torch.bfloat16).to(DEV)
+    gate = randn(g, B, 1, N, dtype=torch.bfloat16).to(DEV)
+    out = torch.empty_like(x)
+    tk.linear_into(a, w, b, out=out.view(M, N), resid=x.view(M, N), gate=gate)
+    gy = gate.float() * oracle.linear_ref_fp32(a, w, b).view(B, L, N)
+    want32 = x.float() + gy
+    bound = 2.0 ** -8 * 1.01 * (2 * gy.abs() + want32.abs()) + 2e-3
+    assert ((out.float() - want32).abs() <= bound).all()

@@ -51,6 +51,7 @@ struct GemmParams {
 };
 
 constexpr int kGemmThreads = 256;
+constexpr int kGemmCUs = 256;      // compute units of the one device this library is built for
 constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
 // A byte offset no buffer of ours reaches (record counts stay below 2^31, and so does k*2 added to
 // it): the buffer load returns zeros for it, which is how rows past M/N and the K tail are padded.
@@ -943,7 +944,39 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     // 256-wide tiles once they fill most of the chip; below that 128-wide ones (two workgroups per
     // CU); problems with too few of those to give every second CU one are bound by the latency of
     // the K loop and run on 64-wide tiles, four times as many workgroups.
-    if (big_tiles >= 160) launch_tiled<4>(p, st);
+    if (big_tiles >= 160) {
+        // One workgroup per CU: a launch whose last round is mostly empty pays for a whole round
+        // (864 tiles of mlp_in at 4608 rows = 3.375 rounds cost 4). When a leading block of whole
+        // tile rows fills whole rounds, it is launched on 256-wide tiles and the few rows left over
+        // follow on 128-wide ones, two workgroups per CU, in one more short round.
+        const int tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+        const int last = static_cast<int>(big_tiles % kGemmCUs);
+        int mb = 0;
+        if (big_tiles > kGemmCUs && last != 0 && last < kGemmCUs / 2) {
+            for (int c = tm - 1; c >= 1 && mb == 0; --c) {
+                const int64_t rest_rows = p.M - static_cast<int64_t>(c) * 256;
+                const int64_t rest_tiles = ((rest_rows + 127) / 128) * ((p.N + 127) / 128);
+                if (rest_tiles > 2 * kGemmCUs) break;
+                const int fill = static_cast<int>((static_cast<int64_t>(c) * tn) % kGemmCUs);
+                if ((fill == 0 || fill >= kGemmCUs * 9 / 10) && (p.gate == nullptr || (c * 256) % p.rows_per_batch == 0)) mb = c;
+            }
+        }
+        if (mb == 0) {
+            launch_tiled<4>(p, st);
+        } else {
+            const int row0 = mb * 256;
+            GemmParams head = p, tail = p;
+            head.M = row0;
+            tail.M = p.M - row0;
+            tail.A += static_cast<int64_t>(row0) * p.lda;
+            tail.Y += static_cast<int64_t>(row0) * p.ldy;
+            if (tail.Y2 != nullptr) tail.Y2 += static_cast<int64_t>(row0) * p.ldy2;
+            if (tail.resid != nullptr) tail.resid += static_cast<int64_t>(row0) * p.ldresid;
+            if (tail.gate != nullptr) tail.gate += static_cast<int64_t>(row0 / p.rows_per_batch) * p.gate_stride;
+            launch_tiled<4>(head, st);
+            launch_tiled<2>(tail, st);
+        }
+    }
     else if (mid_tiles <= 64) launch_tiled<1>(p, st);
     else launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
