@@ -97,9 +97,11 @@ def _time_launches(torch, launches, reps=7):
     return statistics.median(per)
 
 
-def kernel_cases(torch):
+def kernel_cases(torch, extra=False):
     """Yields (name, bound, work, note, build) for every row of the per-kernel table; build() allocates
-    the rotating buffer sets and returns (launches, keepalive)."""
+    the rotating buffer sets and returns (launches, keepalive). extra=True adds rows that only
+    `--only` runs: the same copy and RMSNorm at sixteen times the size, where launch, ramp-up and
+    tail no longer weigh on the rate."""
     import triton_kernels as tk
     from triton_kernels import _native as nv
     from triton_kernels import testing as cfg
@@ -116,7 +118,7 @@ def kernel_cases(torch):
 
     # What a plain device-to-device copy reaches at the sizes of the row-wise kernels below (the
     # practical HBM ceiling of this machine for read-once / write-once traffic, launch included).
-    for mb in (27, 81):
+    for mb in (27, 81, 432) if extra else (27, 81):
         n = mb * 1024 * 1024 // 2
 
         def build(n=n):
@@ -134,6 +136,17 @@ def kernel_cases(torch):
                                                            a.stride(0), a.stride(1), a.stride(2), 0, 0, 1e-6, st)))
                 for a, y in sets], (sets, w)
     yield "rms_norm_qk", "hbm", 2 * (24 * 4608 * 128) * 2 + 256, "", build_rms
+
+    if extra:
+        def build_rms16():
+            x, w = cfg.config1(dev)
+            x = x.expand(16, -1, -1, -1).contiguous()
+            B_, H_, L_, D_ = x.shape
+            sets = [(x.clone(), torch.empty_like(x)) for _ in range(3)]
+            return [(lambda a=a, y=y: check(lib.flux_rms_norm(a.data_ptr(), w.data_ptr(), y.data_ptr(), None, B_, H_, L_, D_,
+                                                               a.stride(0), a.stride(1), a.stride(2), 0, 0, 1e-6, st)))
+                    for a, y in sets], (sets, w)
+        yield "rms_norm_qk_x16", "hbm", 16 * 2 * (24 * 4608 * 128) * 2 + 256, "x [16,24,4608,128]", build_rms16
 
     # C2: LayerNorm + modulation, x [1,4608,3072]
     def build_ln():
@@ -236,7 +249,7 @@ def kernel_table(torch):
 def run_only(torch, which, n_launches):
     """One row of the table by itself: 50 ms of its launches to settle the clocks, then n_launches
     launches inside one event pair. This is the command the rocprofv3 summaries under profiles/ wrap."""
-    for name, bound, work, note, build in kernel_cases(torch):
+    for name, bound, work, note, build in kernel_cases(torch, extra=True):
         if name != which:
             continue
         launches, keep = build()
@@ -254,7 +267,7 @@ def run_only(torch, which, n_launches):
         res = _entry(a.elapsed_time(b) * 1e3 / n_launches, bound, work, note)
         print(json.dumps({"only": name, "launches_timed": n_launches, **res}))
         return
-    names = [c[0] for c in kernel_cases(torch)]
+    names = [c[0] for c in kernel_cases(torch, extra=True)]
     print(f"bench.py --only: unknown kernel {which!r}; one of {names}", file=sys.stderr)
     sys.exit(2)
 
