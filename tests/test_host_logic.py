@@ -1,6 +1,8 @@
 """Host-side behaviour of the Python operator layer that can be checked without a GPU: the public
 names, the exceptions the reference raises, the no-CPU-fallback rule, state-dict compatibility and
 the launch spelling of the raw ops."""
+import os
+
 import pytest
 import torch
 
@@ -115,3 +117,24 @@ def test_seeded_inputs_are_reproducible():
     assert pe.shape == (1, 1, 8, 64, 2, 2) and pe.dtype == torch.float32
     from oracle import flux_oracle as oracle
     assert torch.equal(pe, oracle.embed_nd_ref(oracle.flux_ids(4, 2, 2)))    # package builder == oracle builder
+
+
+def test_bench_reads_traffic_from_the_committed_summary_and_refuses_more_gpus():
+    """bench.py takes roofline.traffic from the counter summary under profiles/ (not from a literal), and
+    a run on more than one GPU exits with a message."""
+    import importlib.util
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    traffic = bench.linear1_traffic_bytes()
+    text = open(os.path.join(root, "profiles", "gemm_linear1_linear2_4608_hbm_traffic.md")).read()
+    line = next(l for l in text.splitlines() if l.startswith("linear1_traffic_bytes_per_launch:"))
+    assert traffic == int(line.split(":")[1].split()[0])
+    algorithmic = 2 * (4608 * 3072 + 21504 * 3072 + 4608 * 21504)          # A, W and Y once, bf16
+    assert algorithmic < traffic < 8 * algorithmic
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
