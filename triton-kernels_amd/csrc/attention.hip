@@ -1057,26 +1057,42 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
     wait_all_vmem();
     mfma_settle();
 
-    // ---- finish: fold the four lane groups' partial sums, normalise, store
+    // ---- finish: fold the four lane groups' partial sums, normalise, store. A lane holds runs of four
+    // columns of sixteen different rows, which would leave as 32-byte pieces; instead the wave parks
+    // its rows in LDS (the rings are idle once every wave is past the loop) and they leave as 16-byte
+    // pieces of whole 256-byte rows. 8-byte slot s of row r sits at slot s ^ 2(r & 15): writes and
+    // reads both spread over all banks, and a 16-byte chunk stays contiguous.
+    asm volatile("s_barrier" ::: "memory");
+    char* const stage = lds + wave * (16 * QB * ROWB);
     static_for<0, QB>([&](auto qb_c) {
         constexpr int qb = decltype(qb_c)::value, QBC = qb;
         float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
         l_tot += __shfl_xor(l_tot, 32, 64);
         const float inv = 1.0f / l_tot;
         const int row = q0 + qb * 16 + r16;
-        if (row < p.L) {
-            bf16_t* orow = p.o + b * p.o_sb + h * p.o_sh + static_cast<int64_t>(row) * p.o_sl;
-            static_for<0, DBN>([&](auto db_c) {
-                constexpr int db = decltype(db_c)::value, r = 4 * (db * QB + QBC);
-                u32x2 w;
-                w.x = pack2_bf16(acc_read<r>() * inv, acc_read<r + 1>() * inv);
-                w.y = pack2_bf16(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
-                *reinterpret_cast<u32x2*>(orow + db * 16 + g * 4) = w;
-            });
-            if (p.lse != nullptr && g == 0)
-                p.lse[static_cast<int64_t>(bh) * p.L + row] = -seed[qb][0] + __builtin_amdgcn_logf(l_tot);
-        }
+        char* const srow = stage + (qb * 16 + r16) * ROWB;
+        static_for<0, DBN>([&](auto db_c) {
+            constexpr int db = decltype(db_c)::value, r = 4 * (db * QB + QBC);
+            u32x2 w;
+            w.x = pack2_bf16(acc_read<r>() * inv, acc_read<r + 1>() * inv);
+            w.y = pack2_bf16(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
+            *reinterpret_cast<u32x2*>(srow + (((db * 4 + g) ^ (r16 * 2)) * 8)) = w;
+        });
+        if (row < p.L && p.lse != nullptr && g == 0)
+            p.lse[static_cast<int64_t>(bh) * p.L + row] = -seed[qb][0] + __builtin_amdgcn_logf(l_tot);
     });
+    __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
+    {
+        bf16_t* const obase = p.o + b * p.o_sb + h * p.o_sh;
+        const int chunk = lane & 15;
+#pragma unroll
+        for (int it = 0; it < 4 * QB; ++it) {
+            const int rl = it * 4 + (lane >> 4);
+            const u32x4 y = *reinterpret_cast<const u32x4*>(stage + rl * ROWB + ((chunk ^ (rl & 15)) * 16));
+            const int row = q0 + rl;
+            if (row < p.L) *reinterpret_cast<u32x4*>(obase + static_cast<int64_t>(row) * p.o_sl + chunk * 8) = y;
+        }
+    }
 }
 
 
