@@ -655,7 +655,7 @@ constexpr int attn_load_slot(int j, int ns, int bs, int sp, bool second) {
 //   <3, 4>: 48 rows per wave, 192 per workgroup: the same code with three quarters of the work per
 //           iteration, for the launch that evens out the last round (see attn_launch_w64).
 template <int QB, int NW>
-__global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) {
+__device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, const int block, const int nblocks) {
     static_assert(NW == 4 && (QB == 3 || QB == 4), "configurations that have been laid out and measured");
     constexpr int ROWS = 16 * QB * NW;         // query rows per workgroup
     constexpr int D = 128, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
@@ -671,10 +671,9 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
     static_assert(BS > 7 * QB - LA && BS < NS - LA, "barrier between the last read of K(T) and the first of K(T+1)");
     static_assert(attn_load_slot(LPW - 1, NS, BS, NS / 8, false) != -2, "load slots");
     constexpr float kRebase = 1.0995116e12f;  // 2^40
-    __shared__ __attribute__((aligned(1024))) char lds[8 * TB];  // K ring of 4 tiles, V ring of 4 tiles
-
-    const int per_xcd = gridDim.x / 8;
-    const int vt = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    // lds: 8 * TB bytes, K ring of 4 tiles, V ring of 4 tiles
+    const int per_xcd = nblocks / 8;
+    const int vt = (block % 8) * per_xcd + block / 8;
     if (vt >= p.total_tiles) return;
     const int per_pair = p.cnt_even + p.cnt_odd;
     const int pair = vt / per_pair, rem = vt % per_pair;
@@ -1096,6 +1095,24 @@ __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) 
 }
 
 
+constexpr int kW64LdsBytes = 8 * 64 * 256;  // K ring and V ring of four 64-key tiles of 256-byte rows
+
+template <int QB, int NW>
+__global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) {
+    __shared__ __attribute__((aligned(1024))) char lds[kW64LdsBytes];
+    attn_w64_tile<QB, NW>(p, lds, blockIdx.x, gridDim.x);
+}
+
+// Both tile sizes in one launch: blocks [0, n4) take 256-row tiles of p4, the rest 192-row tiles of
+// p3. Workgroups are handed out in order, so the 192-row tiles start on each CU as it finishes its
+// 256-row tile, with no launch boundary in between. n4 and the remainder are multiples of eight, so
+// a block's XCD is the same counted from either start.
+__global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel_pair(AttnParams p4, AttnParams p3, int n4) {
+    __shared__ __attribute__((aligned(1024))) char lds[kW64LdsBytes];
+    if (static_cast<int>(blockIdx.x) < n4) attn_w64_tile<4, 4>(p4, lds, blockIdx.x, n4);
+    else attn_w64_tile<3, 4>(p3, lds, static_cast<int>(blockIdx.x) - n4, static_cast<int>(gridDim.x) - n4);
+}
+
 template <int D, int QB, int BN>
 static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
     p.n_qtiles = (p.L + 128 * QB - 1) / (128 * QB);
@@ -1111,18 +1128,18 @@ constexpr int64_t kW64MinTiles = 128;
 // and two rounds it is cut into two launches instead, each at most one round: 256-row tiles for the
 // first rows of every (batch, head), 192-row tiles for the rest, with the cut alternating between
 // even and odd (batch, head) pairs so that both launches come out close to full. 110 592 rows of
-// the Flux shape become 252 + 240 workgroups, 1.75 rounds' worth of time instead of 2.
+// the Flux shape become 252 + 240 workgroups, 1.75 rounds' worth of time instead of 2. The two
+// "launches" are the two block ranges of one kernel (attn_fwd_w64_kernel_pair).
 constexpr int kAttnCUs = 256;
 
-template <int QB>
-static void attn_launch_w64_part(AttnParams p, int64_t BH, int cnt_even, int cnt_odd, int first_even, int first_odd, hipStream_t st) {
+// Fills in the tile mapping of one part and returns its grid (a multiple of eight, 0 = no tiles).
+static int attn_w64_part(AttnParams& p, int64_t BH, int cnt_even, int cnt_odd, int first_even, int first_odd) {
     p.cnt_even = cnt_even; p.cnt_odd = cnt_odd; p.first_even = first_even; p.first_odd = first_odd;
     const int64_t pairs = (BH + 1) / 2;
     p.total_tiles = static_cast<int>(pairs * (cnt_even + cnt_odd));
-    if (p.total_tiles == 0) return;
+    if (p.total_tiles == 0) return 0;
     if (BH % 2) p.total_tiles -= cnt_odd;  // the last pair has no odd member: its tiles sit at the very end
-    const int grid = ((p.total_tiles + 7) / 8) * 8;
-    hipLaunchKernelGGL((attn_fwd_w64_kernel<QB, 4>), dim3(grid), dim3(256), 0, st, p);
+    return ((p.total_tiles + 7) / 8) * 8;
 }
 
 static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
@@ -1140,12 +1157,16 @@ static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
             }
         if (best_ne >= 0) {
             const int fe = min(p.L, best_ne * 256), fo = min(p.L, best_no * 256);
-            attn_launch_w64_part<4>(p, BH, best_ne, best_no, 0, 0, st);
-            attn_launch_w64_part<3>(p, BH, (p.L - fe + 191) / 192, (p.L - fo + 191) / 192, fe, fo, st);
+            AttnParams p4 = p, p3 = p;
+            const int g4 = attn_w64_part(p4, BH, best_ne, best_no, 0, 0);
+            const int g3 = attn_w64_part(p3, BH, (p.L - fe + 191) / 192, (p.L - fo + 191) / 192, fe, fo);
+            if (g3 == 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<4, 4>), dim3(g4), dim3(256), 0, st, p4);
+            else hipLaunchKernelGGL(attn_fwd_w64_kernel_pair, dim3(g4 + g3), dim3(256), 0, st, p4, p3, g4);
             return;
         }
     }
-    attn_launch_w64_part<4>(p, BH, n256, n256, 0, 0, st);
+    const int g = attn_w64_part(p, BH, n256, n256, 0, 0);
+    if (g > 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<4, 4>), dim3(g), dim3(256), 0, st, p);
 }
 
 }  // namespace flux
