@@ -653,7 +653,7 @@ constexpr int attn_load_slot(int j, int ns, int bs, int sp, bool second) {
 // QB = 16-row query blocks per wave, NW = waves per workgroup: 16*QB*NW query rows per workgroup.
 //   <4, 4>: 64 rows per wave, 256 per workgroup, one wave per SIMD (248 vector + 192 accumulation registers).
 //   <3, 4>: 48 rows per wave, 192 per workgroup: the same code with three quarters of the work per
-//           iteration, for the launch that evens out the last round (see attn_launch_w64).
+//           iteration, for the part that evens out the last round (see attn_launch_w64).
 template <int QB, int NW>
 __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, const int block, const int nblocks) {
     static_assert(NW == 4 && (QB == 3 || QB == 4), "configurations that have been laid out and measured");
@@ -1125,11 +1125,11 @@ constexpr int64_t kW64MinTiles = 128;
 
 // One workgroup per CU, so a launch of more than one round's worth of equal tiles costs whole
 // rounds: 432 tiles of 256 rows on 256 CUs take as long as 512 would. When the work is between one
-// and two rounds it is cut into two launches instead, each at most one round: 256-row tiles for the
+// and two rounds it is cut into two parts instead, each at most one round: 256-row tiles for the
 // first rows of every (batch, head), 192-row tiles for the rest, with the cut alternating between
-// even and odd (batch, head) pairs so that both launches come out close to full. 110 592 rows of
+// even and odd (batch, head) pairs so that both parts come out close to full. 110 592 rows of
 // the Flux shape become 252 + 240 workgroups, 1.75 rounds' worth of time instead of 2. The two
-// "launches" are the two block ranges of one kernel (attn_fwd_w64_kernel_pair).
+// parts are the two block ranges of one launch (attn_fwd_w64_kernel_pair).
 constexpr int kAttnCUs = 256;
 
 // Fills in the tile mapping of one part and returns its grid (a multiple of eight, 0 = no tiles).
@@ -1146,7 +1146,7 @@ static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
     const int n256 = (p.L + 255) / 256;
     const int64_t tiles = BH * n256;
     if (tiles > kAttnCUs && tiles <= 2 * kAttnCUs && BH % 2 == 0) {
-        // the most 256-row tiles (ne + no per pair) such that both launches fit one round
+        // the most 256-row tiles (ne + no per pair) such that both parts fit one round
         const int64_t pairs = BH / 2;
         int best_ne = -1, best_no = -1;
         for (int ne = 0; ne <= n256; ++ne)
