@@ -129,3 +129,25 @@ def test_attention_generated_code_uses_no_accumulation_registers_of_its_own():
     if not os.path.exists(path):
         pytest.skip("library not built in this tree")
     assert _isa_checker().check(path) == []
+
+
+def test_gemm_generated_code_does_not_spill(tmp_path):
+    """The tiled GEMM must not touch scratch memory (a spill costs a factor of several in time and nothing
+    in correctness): the checker flags a spill, and the assembly the build keeps passes it."""
+    import importlib.util
+    import pytest
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("check_no_scratch", os.path.join(here, "..", "triton-kernels_amd", "csrc", "check_no_scratch.py"))
+    chk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(chk)
+    good = "_ZN4flux19gemm_nt_ring_kernelILi4ELb0EEEvNS_10GemmParamsE:\n\tv_add_f32_e32 v1, v2, v3\n\ts_endpgm\n"
+    f = tmp_path / "g.s"
+    f.write_text(good)
+    assert chk.check(str(f), "gemm_nt_ring_kernel") == []
+    f.write_text(good.replace("\tv_add_f32_e32 v1, v2, v3", "\tscratch_store_dwordx4 off, v[40:43], off ; 16-byte Folded Spill"))
+    assert len(chk.check(str(f), "gemm_nt_ring_kernel")) == 1
+    assert chk.check(str(f), "no_such_kernel")
+    path = os.path.join(here, "..", "build", "csrc", "gemm_bf16-hip-amdgcn-amd-amdhsa-gfx950.s")
+    if not os.path.exists(path):
+        pytest.skip("library not built in this tree")
+    assert chk.check(path, "gemm_nt_ring_kernel") == []
