@@ -619,7 +619,11 @@ constexpr AttnSched attn_sched() {
         }
     }
     while (head < tail) { S.kind[NS - 1][S.n[NS - 1]] = qk[head]; S.arg[NS - 1][S.n[NS - 1]] = qa[head]; ++S.n[NS - 1]; ++head; }
-    S.kind[NS - 1][S.n[NS - 1]] = ATT_CHECK; S.arg[NS - 1][S.n[NS - 1]] = 0; ++S.n[NS - 1];
+    // The overflow test goes right behind the last add, not into the last slot: the MFMAs and reads
+    // of the slots after it then stand between the compare and the branch that takes its result.
+    int last = NS - 1;
+    while (last > 0 && S.n[last] == 0) --last;
+    S.kind[last][S.n[last]] = ATT_CHECK; S.arg[last][S.n[last]] = 0; ++S.n[last];
     return S;
 }
 template <int QB>
