@@ -127,7 +127,10 @@ _WIDE = [(4, 24, 512),    # 64-row-per-wave kernel, one launch of 256-row tiles
          (3, 24, 1536),   # two launches, odd batch * even heads
          (8, 24, 31),     # one partial tile per head
          (6, 24, 97),
-         (1, 8, 4100)]    # few heads, long ragged sequence
+         (1, 8, 4100),    # few heads, long ragged sequence
+         (2, 43, 770),    # both tile sizes in one launch, ragged, 4 tiles of 256 rows per head
+         (1, 170, 520),   # the same just under two rounds of tiles
+         (257, 1, 257)]   # an odd number of (batch, head) pairs just over two rounds
 
 
 @pytest.mark.parametrize("B,H,L", _WIDE)
