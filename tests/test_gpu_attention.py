@@ -130,7 +130,9 @@ _WIDE = [(4, 24, 512),    # 64-row-per-wave kernel, one launch of 256-row tiles
          (1, 8, 4100),    # few heads, long ragged sequence
          (2, 43, 770),    # both tile sizes in one launch, ragged, 4 tiles of 256 rows per head
          (1, 170, 520),   # the same just under two rounds of tiles
-         (257, 1, 257)]   # an odd number of (batch, head) pairs just over two rounds
+         (257, 1, 257),   # an odd number of (batch, head) pairs just over two rounds
+         (2, 24, 4608),   # 864 tiles of 256 rows = 3.4 rounds: 576 such tiles and 384 of 192 rows
+         (1, 25, 2300)]   # an odd head count with both tile sizes
 
 
 @pytest.mark.parametrize("B,H,L", _WIDE)

@@ -1128,12 +1128,12 @@ static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
 constexpr int64_t kW64MinTiles = 128;
 
 // One workgroup per CU, so a launch of more than one round's worth of equal tiles costs whole
-// rounds: 432 tiles of 256 rows on 256 CUs take as long as 512 would. When the work is between one
-// and two rounds it is cut into two parts instead, each at most one round: 256-row tiles for the
-// first rows of every (batch, head), 192-row tiles for the rest, with the cut alternating between
-// even and odd (batch, head) pairs so that both parts come out close to full. 110 592 rows of
-// the Flux shape become 252 + 240 workgroups, 1.75 rounds' worth of time instead of 2. The two
-// parts are the two block ranges of one launch (attn_fwd_w64_kernel_pair).
+// rounds: 432 tiles of 256 rows on 256 CUs take as long as 512 would. The rows of every (batch, head)
+// are therefore cut in two parts: 256-row tiles for the first rows, 192-row tiles for the rest, with
+// the cut allowed to differ between the even and the odd member of a (batch, head) pair, chosen so
+// that the last workgroup finishes earliest (attn_launch_w64). 110 592 rows of the Flux shape become
+// 252 + 240 workgroups, 1.8 tile times instead of 2. The two parts are the two block ranges of one
+// launch (attn_fwd_w64_kernel_pair).
 constexpr int kAttnCUs = 256;
 
 // Fills in the tile mapping of one part and returns its grid (a multiple of eight, 0 = no tiles).
@@ -1146,26 +1146,51 @@ static int attn_w64_part(AttnParams& p, int64_t BH, int cnt_even, int cnt_odd, i
     return ((p.total_tiles + 7) / 8) * 8;
 }
 
+// When the last 256-row tile has been handed out and all 192-row tiles after it, in units of a fifth
+// of a 256-row tile's time (a 192-row tile takes four: 112 and 90 us measured at the Flux shape).
+// Workgroups are handed out in order to whichever CU is free.
+static int64_t attn_w64_makespan(int64_t n4, int64_t n3) {
+    const int64_t q = n4 / kAttnCUs, r = n4 % kAttnCUs;
+    const int64_t ta = 5 * q, tb = ta + 5;   // kAttnCUs - r CUs are free at ta, the other r at tb
+    const int64_t busy = r ? tb : ta;
+    if (n3 == 0) return busy;
+    auto taken = [&](int64_t t) {  // 192-row tiles finished by time t
+        return (kAttnCUs - r) * (t > ta ? (t - ta) / 4 : 0) + r * (t > tb ? (t - tb) / 4 : 0);
+    };
+    int64_t lo = ta, hi = tb + 4 * (n3 / kAttnCUs + 2);
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) / 2;
+        if (taken(mid) >= n3) hi = mid;
+        else lo = mid + 1;
+    }
+    return lo > busy ? lo : busy;
+}
+
 static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
     const int n256 = (p.L + 255) / 256;
     const int64_t tiles = BH * n256;
-    if (tiles > kAttnCUs && tiles <= 2 * kAttnCUs && BH % 2 == 0) {
-        // the most 256-row tiles (ne + no per pair) such that both parts fit one round
-        const int64_t pairs = BH / 2;
-        int best_ne = -1, best_no = -1;
+    // More than one round of tiles, and few enough rounds for the last one to matter: choose how many
+    // 256-row tiles the even and the odd (batch, head) of a pair get (ne, no; the rest of their rows
+    // goes to 192-row tiles) so that the last workgroup finishes earliest; among equals, the most
+    // 256-row tiles, which are the more efficient ones.
+    if (tiles > kAttnCUs && tiles <= 16 * kAttnCUs && n256 <= 64) {
+        const int64_t pairs = BH / 2, lone = BH % 2;   // a last (batch, head) without a partner counts as an even one
+        int best_ne = n256, best_no = n256;
+        int64_t best_t = attn_w64_makespan(tiles, 0), best_n4 = tiles;
         for (int ne = 0; ne <= n256; ++ne)
             for (int no = ne; no <= n256; ++no) {
                 const int re = p.L - min(p.L, ne * 256), ro = p.L - min(p.L, no * 256);
-                const int64_t w1 = pairs * (ne + no), w2 = pairs * ((re + 191) / 192 + (ro + 191) / 192);
-                if (w1 <= kAttnCUs && w2 <= kAttnCUs && (best_ne < 0 || ne + no > best_ne + best_no)) { best_ne = ne; best_no = no; }
+                const int64_t n4 = pairs * (ne + no) + lone * ne;
+                const int64_t n3 = pairs * ((re + 191) / 192 + (ro + 191) / 192) + lone * ((re + 191) / 192);
+                const int64_t t = attn_w64_makespan(n4, n3);
+                if (t < best_t || (t == best_t && n4 > best_n4)) { best_t = t; best_n4 = n4; best_ne = ne; best_no = no; }
             }
-        if (best_ne >= 0) {
+        if (best_ne < n256 || best_no < n256) {
             const int fe = min(p.L, best_ne * 256), fo = min(p.L, best_no * 256);
             AttnParams p4 = p, p3 = p;
             const int g4 = attn_w64_part(p4, BH, best_ne, best_no, 0, 0);
             const int g3 = attn_w64_part(p3, BH, (p.L - fe + 191) / 192, (p.L - fo + 191) / 192, fe, fo);
-            if (g3 == 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<4, 4>), dim3(g4), dim3(256), 0, st, p4);
-            else hipLaunchKernelGGL(attn_fwd_w64_kernel_pair, dim3(g4 + g3), dim3(256), 0, st, p4, p3, g4);
+            hipLaunchKernelGGL(attn_fwd_w64_kernel_pair, dim3(g4 + g3), dim3(256), 0, st, p4, p3, g4);
             return;
         }
     }
