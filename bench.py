@@ -75,9 +75,11 @@ def parse_args():
 # per-kernel measurements through the C ABI, with rotating buffer sets so that the 256 MB Infinity
 # Cache cannot serve what is reported as HBM traffic
 # --------------------------------------------------------------------------------------------------
-def _time_launches(torch, launches, reps=7):
-    """launches: list of zero-argument callables (one per buffer set), run back to back inside one
-    event pair. Returns the median time per launch in microseconds."""
+def _time_launches(torch, launches, reps=7, min_launches=48):
+    """launches: list of zero-argument callables (one per buffer set). A timed region is at least
+    min_launches launches back to back inside one event pair, cycling through the buffer sets, so
+    that the idle gap in front of a region (synchronisation, event creation) does not weigh on a
+    region of only a few short launches. Returns the median time per launch in microseconds."""
     t_end = time.perf_counter() + 0.05     # warm-up: the clocks settle under sustained load only
     while True:
         for f in launches:
@@ -88,12 +90,14 @@ def _time_launches(torch, launches, reps=7):
     per = []
     for _ in range(reps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        cycles = -(-min_launches // len(launches))
         a.record()
-        for f in launches:
-            f()
+        for _ in range(cycles):
+            for f in launches:
+                f()
         b.record()
         torch.cuda.synchronize()
-        per.append(a.elapsed_time(b) * 1e3 / len(launches))
+        per.append(a.elapsed_time(b) * 1e3 / (cycles * len(launches)))
     return statistics.median(per)
 
 
