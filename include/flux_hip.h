@@ -181,9 +181,12 @@ int flux_linear_bf16(const flux_linear_args* args, void* stream);
  * does not do); any finite sm_scale, negative and zero included. lse (nullable) receives
  * m + log2(l) per row as fp32 [B,H,L], the quantity kernels/attention.py:166-169 stores.
  * For D = 64 and 128 the kernels fold sm_scale * log2(e) into Q and round the result to bf16 once
- * where kernels/attention.py:29-30 scales the fp32 scores: scores, and with them lse, carry that
- * rounding (a few 1e-3 in the base-2 domain for unit-variance inputs; o stays within 2e-2 of the
- * fp32 result). D = 16, 32 and 256 run a plain, unpipelined kernel that scales the fp32 scores.
+ * where kernels/attention.py:29-30 scales the fp32 scores. Every term of a score then carries a
+ * relative error of at most 2^-8, so row i's base-2 scores, and with them lse, move by at most
+ * 2^-8 * sm_scale * log2(e) * max_j sum_d |q_id k_jd|: a few 1e-3 for unit-variance inputs (o within
+ * 4e-3 of the fp32 result at L = 4608), growing in proportion to |q| |k| (q thirty times larger:
+ * lse up to 0.37 away, nearly one-hot outputs up to 0.25 at |v| ~ 4, 1e-2 on average). D = 16, 32
+ * and 256 run a plain, unpipelined kernel that scales the fp32 scores.
  * ------------------------------------------------------------------------------------------- */
 typedef struct flux_attn_args {
     flux_src4 q, k, v;

@@ -30,6 +30,7 @@
 #include "common.h"
 #include "attention_params.h"
 #include <stdlib.h>
+#include <mutex>
 #include <type_traits>
 
 namespace flux {
@@ -70,7 +71,7 @@ __device__ __forceinline__ void lds_load16_raw(u32x4 rsrc, uint32_t lds_addr, ui
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
-                 : "memory");  // m0 is written: a register the compiler reserves and never allocates on this target
+                 : "memory", "m0");
 }
 // The same with the LDS address given as a scalar base plus a constant.
 template <int OFF>
@@ -78,7 +79,7 @@ __device__ __forceinline__ void lds_load16_raw_at(u32x4 rsrc, uint32_t lds_base,
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
                  : "s"(lds_base), "v"(voff), "s"(rsrc), "n"(OFF)
-                 : "memory", "scc");  // and m0, see above
+                 : "memory", "scc", "m0");
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p));
@@ -1017,22 +1018,24 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     // per body; the record count is what is left of the sequence, at most one tile.
     uint64_t k_at = reinterpret_cast<uint64_t>(kbase) + static_cast<uint64_t>(4 * 64) * k_row2;
     uint64_t v_at = reinterpret_cast<uint64_t>(vbase) + static_cast<uint64_t>(2 * 64) * v_row2;
-    int k_left = (p.L - 4 * 64 - 1) * k_row2 + D * 2, v_left = (p.L - 2 * 64 - 1) * v_row2 + D * 2;  // bytes up to the end of the last row
-    const int k_tile = 63 * k_row2 + D * 2, v_tile = 63 * v_row2 + D * 2;
-    auto next_rsrc = [&](uint64_t& at, int& left, int step, int tile) -> u32x4 {
+    // rows left from the start of the next tile to request; a tile's record count is formed from at most
+    // 64 of them, so it stays in 32 bits however long and widely strided the sequence is
+    int k_rows = p.L - 4 * 64, v_rows = p.L - 2 * 64;
+    auto next_rsrc = [&](uint64_t& at, int& rows_left, int row2) -> u32x4 {
+        const int rows = min(rows_left, 64);
         u32x4 r;
         r.x = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at));
         r.y = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at >> 32) & 0xffffu);
-        r.z = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max(min(left, tile), 0)));
+        r.z = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(rows > 0 ? (rows - 1) * row2 + D * 2 : 0));
         r.w = kAttnRsrcFlags;
-        at += static_cast<uint64_t>(step);
-        left -= step;
+        at += static_cast<uint64_t>(64) * static_cast<uint64_t>(row2);
+        rows_left -= 64;
         return r;
     };
     auto body = [&](auto r_c, auto rag_c, int T) -> bool {
         constexpr int r = decltype(r_c)::value, r0 = r * TB, r1 = ((r + 1) & 3) * TB, r2 = ((r + 2) & 3) * TB, r3 = ((r + 3) & 3) * TB;
         using ic = std::integral_constant<int, 0>;
-        const u32x4 rk = next_rsrc(k_at, k_left, 64 * k_row2, k_tile), rv = next_rsrc(v_at, v_left, 64 * v_row2, v_tile);
+        const u32x4 rk = next_rsrc(k_at, k_rows, k_row2), rv = next_rsrc(v_at, v_rows, v_row2);
         iter(std::true_type{}, rag_c, std::integral_constant<int, r0 + HALF>{}, std::integral_constant<int, r1>{},
              std::integral_constant<int, r3 + HALF>{}, std::integral_constant<int, r0>{}, std::integral_constant<int, r2>{},
              rk, rv, 2 * T, s0, s1, pw0, pw1);
@@ -1166,6 +1169,38 @@ static int64_t attn_w64_makespan(int64_t n4, int64_t n3) {
     return lo > busy ? lo : busy;
 }
 
+// The cut that attn_launch_w64 uses for BH (batch, head)s of L rows: ne / no = 256-row tiles of the even
+// and the odd member of a pair. The search below evaluates up to a few thousand makespans, so the last
+// few answers are kept (a serving loop calls with the same one or two shapes over and over).
+static void attn_w64_cut(int64_t BH, int L, int& best_ne, int& best_no) {
+    struct Entry { int64_t BH; int L, ne, no; };
+    static std::mutex mu;
+    static Entry cache[8];
+    static int filled = 0, next = 0;
+    {
+        std::lock_guard<std::mutex> g(mu);
+        for (int i = 0; i < filled; ++i)
+            if (cache[i].BH == BH && cache[i].L == L) { best_ne = cache[i].ne; best_no = cache[i].no; return; }
+    }
+    const int n256 = (L + 255) / 256;
+    const int64_t tiles = BH * n256;
+    const int64_t pairs = BH / 2, lone = BH % 2;   // a last (batch, head) without a partner counts as an even one
+    best_ne = n256; best_no = n256;
+    int64_t best_t = attn_w64_makespan(tiles, 0), best_n4 = tiles;
+    for (int ne = 0; ne <= n256; ++ne)
+        for (int no = ne; no <= n256; ++no) {
+            const int re = L - min(L, ne * 256), ro = L - min(L, no * 256);
+            const int64_t n4 = pairs * (ne + no) + lone * ne;
+            const int64_t n3 = pairs * ((re + 191) / 192 + (ro + 191) / 192) + lone * ((re + 191) / 192);
+            const int64_t t = attn_w64_makespan(n4, n3);
+            if (t < best_t || (t == best_t && n4 > best_n4)) { best_t = t; best_n4 = n4; best_ne = ne; best_no = no; }
+        }
+    std::lock_guard<std::mutex> g(mu);
+    cache[next] = Entry{BH, L, best_ne, best_no};
+    next = (next + 1) % 8;
+    if (filled < 8) ++filled;
+}
+
 static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
     const int n256 = (p.L + 255) / 256;
     const int64_t tiles = BH * n256;
@@ -1174,17 +1209,8 @@ static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
     // goes to 192-row tiles) so that the last workgroup finishes earliest; among equals, the most
     // 256-row tiles, which are the more efficient ones.
     if (tiles > kAttnCUs && tiles <= 16 * kAttnCUs && n256 <= 64) {
-        const int64_t pairs = BH / 2, lone = BH % 2;   // a last (batch, head) without a partner counts as an even one
-        int best_ne = n256, best_no = n256;
-        int64_t best_t = attn_w64_makespan(tiles, 0), best_n4 = tiles;
-        for (int ne = 0; ne <= n256; ++ne)
-            for (int no = ne; no <= n256; ++no) {
-                const int re = p.L - min(p.L, ne * 256), ro = p.L - min(p.L, no * 256);
-                const int64_t n4 = pairs * (ne + no) + lone * ne;
-                const int64_t n3 = pairs * ((re + 191) / 192 + (ro + 191) / 192) + lone * ((re + 191) / 192);
-                const int64_t t = attn_w64_makespan(n4, n3);
-                if (t < best_t || (t == best_t && n4 > best_n4)) { best_t = t; best_n4 = n4; best_ne = ne; best_no = no; }
-            }
+        int best_ne, best_no;
+        attn_w64_cut(BH, p.L, best_ne, best_no);
         if (best_ne < n256 || best_no < n256) {
             const int fe = min(p.L, best_ne * 256), fo = min(p.L, best_no * 256);
             AttnParams p4 = p, p3 = p;
