@@ -275,17 +275,34 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x4 (&
     char* dst_u = reinterpret_cast<char*>(to_y ? p.Y + wave_n0 : p.Y2 + (wave_n0 - p.split_n + p.y2_col0));
     const int64_t dst_ld = (to_y ? p.ldy : p.ldy2) * 2;            // bytes
     const uint32_t dst_lane = static_cast<uint32_t>(rrow * dst_ld + rch * 16);
+    // Gated residual: the rows of resid this lane adds to are requested a whole 32-row block ahead,
+    // into the other half of rs, so that they land while the block in front is converted and stored.
+    // (Requested where they are used, every 16-byte store waited for a load round trip of its own,
+    // and, the memory counter being in-order, for the store in front of it: 32 round trips in a row
+    // per wave.) The tile lies inside one batch element (the caller checks), so the gate vector of
+    // this lane's eight columns is loaded once.
     const char* res_u = nullptr;
-    const char* gate_u = nullptr;
     uint32_t res_lane = 0;
+    Vec16<bf16_t> gt;
+    Vec16<bf16_t> rs[2][NIT];
+    auto request_resid = [&](int i) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+            rs[i & 1][it] = *reinterpret_cast<const Vec16<bf16_t>*>(res_u + static_cast<int64_t>(wave_m0 + i * 32 + it * RPI) * p.ldresid * 2 + res_lane);
+    };
     if (GATE) {
         res_u = reinterpret_cast<const char*>(p.resid + wave_n0);
         res_lane = static_cast<uint32_t>(rrow * p.ldresid * 2 + rch * 16);
-        gate_u = reinterpret_cast<const char*>(p.gate + wave_n0 + rch * 8);
+        gt = ld16(p.gate + static_cast<int64_t>(m0 / p.rows_per_batch) * p.gate_stride + wave_n0 + rch * 8);
+        request_resid(0);
     }
 
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
+        if (GATE) {
+            if (i + 1 < MI) request_resid(i + 1);
+            __builtin_amdgcn_sched_barrier(0);   // the loads stay in front of the conversion below
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -305,13 +322,11 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x4 (&
             Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + (i * 32 + (it / NSW) * NSW * RPI) * C_PITCH + raddr[it % NSW]);
             const int64_t m_u = wave_m0 + row_u;
             if (GATE) {
-                // all rows of one access belong to one batch element when rows_per_batch is a multiple of RPI
-                const Vec16<bf16_t> gt = ld16(reinterpret_cast<const bf16_t*>(gate_u) + ((m_u + rrow) / p.rows_per_batch) * p.gate_stride);
-                const Vec16<bf16_t> rs = *reinterpret_cast<const Vec16<bf16_t>*>(res_u + m_u * p.ldresid * 2 + res_lane);
+                const Vec16<bf16_t> r = rs[i & 1][it];
 #pragma unroll
                 for (int e = 0; e < 8; e += 2) {
-                    const float y0 = bf2f(rs.v[e]) + bf2f(f2bf(bf2f(gt.v[e]) * bf2f(y.v[e])));
-                    const float y1 = bf2f(rs.v[e + 1]) + bf2f(f2bf(bf2f(gt.v[e + 1]) * bf2f(y.v[e + 1])));
+                    const float y0 = bf2f(r.v[e]) + bf2f(f2bf(bf2f(gt.v[e]) * bf2f(y.v[e])));
+                    const float y1 = bf2f(r.v[e + 1]) + bf2f(f2bf(bf2f(gt.v[e + 1]) * bf2f(y.v[e + 1])));
                     const uint32_t w = pack2_bf16(y0, y1);
                     y.v[e] = static_cast<bf16_t>(w & 0xffffu);
                     y.v[e + 1] = static_cast<bf16_t>(w >> 16);
@@ -464,7 +479,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[
             return;
         }
     }
+    // (with a gate: the fast path loads one gate vector per tile, so the tile must not span batch elements)
     const bool fast = p.vec_io && m0 + BM <= p.M && n0 + BN <= p.N && (gelu_all || gelu_none) &&
+                      (p.gate == nullptr || m0 / p.rows_per_batch == (m0 + BM - 1) / p.rows_per_batch) &&
                       (wave_n0 + WCOLS <= p.split_n || wave_n0 >= p.split_n) && (p.bias == nullptr || p.bias_vec) &&
                       static_cast<int64_t>(BM) * p.ldy * 2 < 0x7fffffffLL && static_cast<int64_t>(BM) * p.ldy2 * 2 < 0x7fffffffLL;
     if (fast) {
