@@ -35,6 +35,7 @@ METRIC = "Flux single-block ms @4608 tok bf16; per-kernel GB/s & TFLOP/s vs roof
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 BLOCK_GFLOP = 1304.65       # linear1 + attention + linear2 + modulation projection
+SWEEP_MULTS = (1, 2, 4, 8, 16)
 LINEAR1_FLOP = 2.0 * 4608 * 21504 * 3072
 
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemm_linear1_linear2_4608_hbm_traffic.md")
@@ -62,8 +63,12 @@ def parse_args():
     ap.add_argument("--settle-ms", type=float, default=80.0, help="untimed block passes for this long before the warm-up")
     ap.add_argument("--only", default=None, help="run one row of the per-kernel table by itself, then exit")
     ap.add_argument("--launches", type=int, default=20, help="launches timed with --only")
+    ap.add_argument("--sweep", action="store_true",
+                    help="row-wise kernels and a hand-written copy at 1, 2, 4, 8 and 16 times the Flux shape, with the "
+                         "least-squares fit t = t0 + bytes / rate per kernel; then exit")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-graph", action="store_true", help="skip the captured-graph replay of the same block")
     ap.add_argument("--json-out", default=None, help="also write the result, indented, to this file")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain device-to-device copies of 256 MiB (reference for scaling FETCH_SIZE / "
@@ -141,16 +146,19 @@ def kernel_cases(torch, extra=False):
                 for a, y in sets], (sets, w)
     yield "rms_norm_qk", "hbm", 2 * (24 * 4608 * 128) * 2 + 256, "", build_rms
 
+    # The same kernels on 2, 4, 8 and 16 times the rows (batch 2 .. 16), for the fit t = t0 + bytes / rate
+    # that separates launch, ramp-up and tail from the steady rate (--sweep, --only).
     if extra:
-        def build_rms16():
-            x, w = cfg.config1(dev)
-            x = x.expand(16, -1, -1, -1).contiguous()
-            B_, H_, L_, D_ = x.shape
-            sets = [(x.clone(), torch.empty_like(x)) for _ in range(3)]
-            return [(lambda a=a, y=y: check(lib.flux_rms_norm(a.data_ptr(), w.data_ptr(), y.data_ptr(), None, B_, H_, L_, D_,
-                                                               a.stride(0), a.stride(1), a.stride(2), 0, 0, 1e-6, st)))
-                    for a, y in sets], (sets, w)
-        yield "rms_norm_qk_x16", "hbm", 16 * 2 * (24 * 4608 * 128) * 2 + 256, "x [16,24,4608,128]", build_rms16
+        for mult in SWEEP_MULTS[1:]:
+            def build_rms_n(mult=mult):
+                x, w = cfg.config1(dev)
+                x = x.expand(mult, -1, -1, -1).contiguous()
+                B_, H_, L_, D_ = x.shape
+                sets = [(x.clone(), torch.empty_like(x)) for _ in range(n_sets(2 * x.numel() * 2))]
+                return [(lambda a=a, y=y: check(lib.flux_rms_norm(a.data_ptr(), w.data_ptr(), y.data_ptr(), None, B_, H_, L_, D_,
+                                                                   a.stride(0), a.stride(1), a.stride(2), 0, 0, 1e-6, st)))
+                        for a, y in sets], (sets, w)
+            yield f"rms_norm_qk_x{mult}", "hbm", mult * 2 * (24 * 4608 * 128) * 2 + 256, f"x [{mult},24,4608,128]", build_rms_n
 
     # C2: LayerNorm + modulation, x [1,4608,3072]
     def build_ln():
@@ -161,13 +169,26 @@ def kernel_cases(torch, extra=False):
                 for a, y in sets], (sets, sc, sh)
     yield "layer_norm_modulation", "hbm", 2 * (4608 * 3072) * 2 + 2 * 3072 * 2, "", build_ln
 
+    if extra:
+        for mult in SWEEP_MULTS[1:]:
+            def build_ln_n(mult=mult):
+                x, sc, sh = cfg.config2(dev)
+                x = x.expand(mult, -1, -1).contiguous()
+                sc, sh = sc.expand(mult, -1, -1).contiguous(), sh.expand(mult, -1, -1).contiguous()
+                sets = [(x.clone(), torch.empty_like(x)) for _ in range(n_sets(2 * x.numel() * 2))]
+                return [(lambda a=a, y=y: check(lib.flux_layer_norm_modulation(a.data_ptr(), sc.data_ptr(), sh.data_ptr(), y.data_ptr(),
+                                                                                mult, x.shape[1], x.shape[2], x.shape[2], 0, 1e-6, st)))
+                        for a, y in sets], (sets, sc, sh)
+            yield (f"layer_norm_modulation_x{mult}", "hbm", mult * (2 * (4608 * 3072) * 2 + 2 * 3072 * 2), f"x [{mult},4608,3072]",
+                   build_ln_n)
+
     # C3: RoPE alone, concat alone, RoPE + concat fused (argument structs are prepared once per buffer set)
     Lt, Li = 512, 4096
     Ltot = Lt + Li
     qk_elems = 24 * Ltot * 128
     pe_bytes = Ltot * 64 * 4 * 4
 
-    def prep_args(pe, tq, tk_, tv, iq, ik, iv, oq, ok, ov, with_pe, lt):
+    def prep_args(pe, tq, tk_, tv, iq, ik, iv, oq, ok, ov, with_pe, lt, batch=1):
         a = nv.QkvPrepArgs()
         for name, t_, i_, o_ in (("q", tq, iq, oq), ("k", tk_, ik, ok), ("v", tv, iv, ov)):
             if o_ is None:
@@ -178,7 +199,7 @@ def kernel_cases(torch, extra=False):
             setattr(a, f"{name}_out", o_.data_ptr())
         if with_pe:
             a.pe = pe.data_ptr()
-        a.B, a.H, a.Lt, a.Li, a.D = 1, 24, lt, Ltot - lt, 128
+        a.B, a.H, a.Lt, a.Li, a.D = batch, 24, lt, Ltot - lt, 128
         a.dtype = a.scale_dtype = 0
         a.eps = 1e-6
         return a
@@ -212,6 +233,36 @@ def kernel_cases(torch, extra=False):
             return launches, keep
         yield name, "hbm", work, "", build
 
+    if extra:
+        # the fused RoPE + concat at 2 .. 16 times the rows, and the same gather kernel as a plain copy of
+        # q alone (no table, no norm): a hand-written copy of the same structure as the row-wise kernels
+        for mult in SWEEP_MULTS[1:]:
+            def build_fused_n(mult=mult):
+                txt, img, pe = cfg.config3(dev)
+                keep, launches = [pe], []
+                for _ in range(n_sets(mult * 6 * qk_elems * 2)):
+                    t_ = [t.expand(mult, -1, -1, -1).contiguous() for t in txt]
+                    i_ = [t.expand(mult, -1, -1, -1).contiguous() for t in img]
+                    o_ = [torch.empty(mult, 24, Ltot, 128, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+                    a = prep_args(pe, t_[0], t_[1], t_[2], i_[0], i_[1], i_[2], o_[0], o_[1], o_[2], True, Lt, batch=mult)
+                    keep.append((t_, i_, o_, a))
+                    launches.append(lambda a=a: check(lib.flux_qkv_prep(ctypes.byref(a), st)))
+                return launches, keep
+            yield f"rope_concat_fused_x{mult}", "hbm", mult * 6 * qk_elems * 2 + pe_bytes, f"batch {mult}", build_fused_n
+        for mult in SWEEP_MULTS:
+            def build_copy_n(mult=mult):
+                x, _ = cfg.config1(dev)
+                keep, launches = [], []
+                for _ in range(n_sets(mult * 2 * qk_elems * 2)):
+                    q_ = x.expand(mult, -1, -1, -1).contiguous()
+                    oq = torch.empty_like(q_)
+                    a = prep_args(None, None, None, None, q_, None, None, oq, None, None, False, 0, batch=mult)
+                    keep.append((q_, oq, a))
+                    launches.append(lambda a=a: check(lib.flux_qkv_prep(ctypes.byref(a), st)))
+                return launches, keep
+            yield (f"hand_copy_x{mult}", "hbm", mult * 2 * qk_elems * 2,
+                   f"flux_qkv_prep as a plain copy of q [{mult},24,4608,128] (no table, no norm)", build_copy_n)
+
     # C4 / C5: GEMMs (MFMA-bound; three rotating sets keep operands out of L2 between launches)
     for name, which, act, (M, N, K) in (("linear_mlp_in_gelu", "mlp_in", "GELU", (4608, 12288, 3072)),
                                         ("linear_proj_out", "proj_out", "", (4608, 3072, 15360)),
@@ -230,6 +281,42 @@ def kernel_cases(torch, extra=False):
         sets = [(q.clone(), k.clone(), v.clone(), torch.empty_like(q)) for _ in range(3)]
         return [(lambda s=s: tk.attention_into(s[0], s[1], s[2], s[3])) for s in sets], sets
     yield "attention_fwd", "mfma", 4.0 * 24 * 4608 * 4608 * 128, "", build_attn
+
+    # the same launch on the views the fused block passes: v read in place inside the qkv projection
+    # (row stride 9216 elements), o written in "L (H D)" order into the [L, 15360] buffer linear2 reads
+    def build_attn_views():
+        q, k, v = cfg.config5_attention(dev)
+        sets = []
+        for _ in range(3):
+            qkv = torch.empty(1, 4608, 3 * 3072, dtype=torch.bfloat16, device=dev)
+            v_view = qkv.view(1, 4608, 3, 24, 128).permute(2, 0, 3, 1, 4)[2]
+            v_view.copy_(v)
+            both = torch.empty(1, 4608, 3072 + 12288, dtype=torch.bfloat16, device=dev)
+            o_view = both[..., :3072].view(1, 4608, 24, 128).permute(0, 2, 1, 3)
+            sets.append((q.clone(), k.clone(), v_view, o_view, qkv, both))
+        return [(lambda s=s: tk.attention_into(s[0], s[1], s[2], s[3])) for s in sets], sets
+    yield ("attention_fwd_block_views", "mfma", 4.0 * 24 * 4608 * 4608 * 128,
+           "v at row stride 9216 inside qkv, o at row stride 15360 into the concat buffer, as in the fused block", build_attn_views)
+
+    # head dim 64 at the same hidden size (the reference's test grid is D in {64, 128}, tests/test_attention.py:7-21)
+    def build_attn64():
+        g = torch.Generator().manual_seed(1064)
+        mk = lambda: torch.randn((1, 48, 4608, 64), generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        sets = [(mk(), mk(), mk(), torch.empty(1, 48, 4608, 64, dtype=torch.bfloat16, device=dev)) for _ in range(3)]
+        return [(lambda s=s: tk.attention_into(s[0], s[1], s[2], s[3])) for s in sets], sets
+    yield "attention_fwd_d64", "mfma", 4.0 * 48 * 4608 * 4608 * 64, "B1 H48 L4608 D64", build_attn64
+
+    # linear2 as the block runs it: bias and the gated residual x + gate * y in the epilogue, the
+    # residual rows cold (twelve rotating copies, more than the Infinity Cache holds)
+    def build_lin2_gated():
+        a_, w_, b_ = cfg.config4(dev, "proj_out")
+        g = torch.Generator().manual_seed(1077)
+        gate = (torch.randn((1, 1, 3072), generator=g) * 0.5).to(torch.bfloat16).to(dev)
+        xs = [torch.randn((4608, 3072), generator=g).to(torch.bfloat16).to(dev) for _ in range(12)]
+        outs = [torch.empty(4608, 3072, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+        return [(lambda i=i: tk.linear_into(a_, w_, b_, out=outs[i % 3], resid=xs[i], gate=gate)) for i in range(12)], (a_, w_, b_, xs, outs, gate)
+    yield ("linear2_gated_residual", "mfma", 2.0 * 4608 * 3072 * 15360,
+           "proj_out with the block's epilogue: bias, then x + gate * y", build_lin2_gated)
 
 
 def _entry(us, bound, work, note=""):
@@ -276,6 +363,34 @@ def run_only(torch, which, n_launches):
     sys.exit(2)
 
 
+def run_sweep(torch):
+    """Times the row-wise kernels and the hand-written copy at every size of SWEEP_MULTS and fits
+    t = t0 + bytes / rate: t0 is what a launch costs whatever its size (launch, ramp-up, tail), rate the
+    steady HBM rate of the kernel. Prints one JSON object."""
+    fams = {"rms_norm_qk": [], "layer_norm_modulation": [], "rope_concat_fused": [], "hand_copy": []}
+    for name, bound, work, note, build in kernel_cases(torch, extra=True):
+        fam = next((f for f in fams if name == f or name.startswith(f + "_x")), None)
+        if fam is None:
+            continue
+        launches, keep = build()
+        us = _time_launches(torch, launches, reps=5, min_launches=24)
+        fams[fam].append((work, us))
+        del launches, keep
+        torch.cuda.empty_cache()
+    out = {}
+    for fam, pts in fams.items():
+        pts.sort()
+        n = len(pts)
+        sx, sy = sum(b for b, _ in pts), sum(t for _, t in pts)
+        sxx, sxy = sum(b * b for b, _ in pts), sum(b * t for b, t in pts)
+        slope = (n * sxy - sx * sy) / (n * sxx - sx * sx)      # us per byte
+        t0 = (sy - slope * sx) / n
+        rate = 1.0 / slope / 1e3                                 # GB/s
+        out[fam] = {"points": [{"bytes": b, "us": round(t, 2), "GBps": round(b / t / 1e3, 1)} for b, t in pts],
+                    "t0_us": round(t0, 2), "steady_GBps": round(rate, 1), "steady_frac_of_peak": round(rate / HBM_PEAK_GBS, 4)}
+    print(json.dumps({"sweep": out}))
+
+
 # --------------------------------------------------------------------------------------------------
 # CPU baseline: the oracle's single-stream block on the host cores (reported, not a target)
 # --------------------------------------------------------------------------------------------------
@@ -297,6 +412,42 @@ def cpu_baseline(torch):
         "sample": "oracle single_stream_block_ref (plain PyTorch, bf16) on the same seeded 4608-token inputs: "
                   "1 warm-up + 3 timed passes, median; host has %d logical CPUs" % (os.cpu_count() or 0),
     }
+
+
+def graph_replay(torch, blk, x, vec, pe, y_eager, steps):
+    """The same block pass captured once into a HIP graph and replayed `steps` times: what the launch
+    gaps of the eager pass cost. Not the headline (that stays the eager number). The library allocates
+    nothing and records no memset, so capture is legal; every replay is compared with the eager result."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(3):
+                blk(x, vec, pe)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(g):
+            y_g = blk(x, vec, pe)
+        worst = 0.0
+        for _ in range(3):   # replays with eager work and synchronisations in between, each one checked
+            g.replay()
+            torch.cuda.synchronize()
+            worst = max(worst, (y_g.float() - y_eager.float()).abs().max().item())
+            with torch.no_grad():
+                blk(x, vec, pe)
+            torch.cuda.synchronize()
+        for _ in range(10):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        return {"ms_per_step": round(ms, 4), "steps": steps, "max_abs_diff_vs_eager": worst}
+    except Exception as e:  # capture is an extra: report why it did not run, keep the headline
+        return {"error": f"{type(e).__name__}: {e}"[:300]}
 
 
 def main():
@@ -328,6 +479,9 @@ def main():
     if args.only:
         run_only(torch, args.only, args.launches)
         return
+    if args.sweep:
+        run_sweep(torch)
+        return
 
     x, vec, pe, sd = cfg.config5_block(dev)
     blk = tk.SingleStreamBlock(3072, 24).to(torch.bfloat16).to(dev)
@@ -336,7 +490,7 @@ def main():
     # Events around the stages of the fused forward inside the timed steps, through the hook the module
     # exposes for this. They are recorded on torch's current stream, which is the stream every HIP
     # kernel here is launched on. linear1 (N = 21504) is the dominant kernel.
-    stage_events = {"linear1": [], "attention": [], "linear2": []}
+    stage_events = {"modulation": [], "layer_norm": [], "linear1": [], "attention": [], "linear2": []}
     open_ev = {}
 
     def hook(stage, edge):
@@ -369,6 +523,9 @@ def main():
         blk.stage_hook = None
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     stage_us = {k: statistics.mean(e0.elapsed_time(e1) for e0, e1 in v) * 1e3 for k, v in stage_events.items()}
+    # what the five stages leave of a pass: launch gaps between dependent kernels, event records, allocator calls
+    gap_us = ms_per_step * 1e3 - sum(stage_us.values())
+    graph = None if args.no_graph else graph_replay(torch, blk, x, vec, pe, y, args.steps)
     l1_us = stage_us["linear1"]
     l1_tflops = LINEAR1_FLOP / l1_us / 1e6
     assert torch.isfinite(y.float()).all()
@@ -399,7 +556,11 @@ def main():
             "launch_us": round(l1_us, 1), "launches_timed": len(stage_events["linear1"]),
         },
         "block_stage_us": {k: round(v, 1) for k, v in stage_us.items()},
+        "launch_gap_us": round(gap_us, 1),
+        "launch_gap_share": round(gap_us / (ms_per_step * 1e3), 4),
     }
+    if graph is not None:
+        result["graph_replay"] = graph
     if not args.no_kernels:
         result["kernels"] = kernel_table(torch)
     if not args.no_cpu:

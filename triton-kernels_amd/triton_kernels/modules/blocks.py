@@ -164,8 +164,9 @@ class SingleStreamBlock(nn.Module):
     # multiple of 256); otherwise, or with this switched off, one preparation kernel behind linear1
     fuse_qk_epilogue = True
     # Optional callable(stage, edge), invoked on the launching thread right before (edge "begin") and
-    # right after ("end") the launch of a stage of the fused forward: "linear1", "attention",
-    # "linear2". Benchmarks set it to record stream events around a kernel inside real block passes.
+    # right after ("end") the launch of a stage of the forward: "modulation", "layer_norm" and, in the
+    # fused forward, "linear1", "attention", "linear2". Benchmarks set it to record stream events
+    # around a kernel inside real block passes.
     stage_hook = None
 
     def __init__(self, hidden_size: int, num_heads: int, mlp_ratio: float = 4.0, qk_scale: float | None = None):
@@ -183,8 +184,13 @@ class SingleStreamBlock(nn.Module):
         self.modulation = Modulation(hidden_size, double=False)
 
     def forward(self, x: Tensor, vec: Tensor, pe: Tensor) -> Tensor:
+        hook = self.stage_hook or (lambda stage, edge: None)
+        hook("modulation", "begin")
         mod, _ = self.modulation(vec)
+        hook("modulation", "end")
+        hook("layer_norm", "begin")
         x_mod = layer_norm_modulation(x, mod.scale, mod.shift)
+        hook("layer_norm", "end")
         if self.fused and _fusable(x, self.linear1.weight, self.linear2.weight, self.norm.query_norm.scale):
             return self._forward_fused(x, x_mod, mod, pe)
         hid = self.hidden_size
