@@ -151,3 +151,4 @@ def test_gemm_generated_code_does_not_spill(tmp_path):
     if not os.path.exists(path):
         pytest.skip("library not built in this tree")
     assert chk.check(path, "gemm_nt_ring_kernel") == []
+    assert chk.check(path, "gemm_nt_rect_kernel") == []

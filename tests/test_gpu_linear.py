@@ -72,6 +72,39 @@ def test_linear_ragged_shapes(M, N, K, bias):
     assert ((y.float() - ref32).abs() <= half_ulp_bound(ref32)).all()
 
 
+@pytest.mark.parametrize("B,L,N,K,act,bias,gated", [
+    (1, 4608, 3072, 512, "", True, True),       # linear2's output shape: 256 tiles of 288 x 192, gated residual
+    (2, 1152, 6144, 200, "", False, True),      # K tail, two batch elements of four tile rows each, no bias
+    (1, 2304, 6144, 136, "GELU", True, False),  # GELU on every column
+    (1, 2304, 6144, 64, "", True, False),       # a single slab
+    (1, 4608, 3072, 8, "", True, False),        # less than a slab
+])
+def test_linear_rectangular_tiles(B, L, N, K, act, bias, gated):
+    """Shapes that both 288 and 192 divide and that fill the 256 CUs better on 288 x 192 tiles than on
+    square ones take the rectangular-tile kernel: every epilogue it has, with and without a K tail."""
+    g = seeded(B * L + N + K)
+    M = B * L
+    a = randn(g, M, K, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, N, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16, std=0.5).to(DEV) if bias else None
+    ref32 = oracle.linear_ref_fp32(a, w, b, act)
+    if not gated:
+        y = tk.linear(a, w, b, activation=act)
+        assert ((y.float() - ref32).abs() <= half_ulp_bound(ref32)).all()
+        return
+    x = randn(g, B, L, N, dtype=torch.bfloat16).to(DEV)
+    gate = randn(g, B, 1, N, dtype=torch.bfloat16).to(DEV)
+    out = torch.empty_like(x)
+    tk.linear_into(a, w, b, out=out.view(M, N), resid=x.view(M, N), gate=gate)
+    gy = gate.float() * ref32.view(B, L, N)
+    want32 = x.float() + gy
+    bound = 2.0 ** -8 * 1.01 * (2 * gy.abs() + want32.abs()) + 2e-3
+    assert ((out.float() - want32).abs() <= bound).all()
+    # and exactly the two PyTorch ops on the kernel's own (once rounded) product
+    y = tk.linear(a, w, b)
+    assert torch.equal(out, oracle.gated_residual_ref(x, gate, y.view(B, L, N)))
+
+
 def test_linear_unaligned_k_and_strided_input():
     g = seeded(3)
     x = randn(g, 50, 77, dtype=torch.bfloat16).to(DEV)       # K = 77: no 16-byte rows

@@ -735,6 +735,293 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Rectangular tiles: (32*FM) x (32*FN) per workgroup, a wave owns (16*FM) x (16*FN) as FM x FN
+// accumulators. One workgroup per CU means a launch costs whole rounds of 256 tiles; 4608 x 3072
+// (linear2 of the Flux block) is 216 tiles of 256 x 256, 0.84 of a round with 40 CUs idle, but
+// exactly 256 tiles of 288 x 192 (FM = 9, FN = 6: 216 accumulation registers). The main loop is the
+// one above with the two operands' slabs in rings of their own, because their units now differ in
+// size: three units of A (BM rows x 128 bytes) and two of W (BN rows), 156 KB. While slab kt is
+// multiplied, A(kt+1), W(kt+1) and A(kt+2) occupy the other units; behind the barrier of slab kt the
+// unit of W(kt) takes W(kt+2), and the loads of A(kt+3) go into the unit of A(kt) in front of the
+// next barrier. A step has FM + FN fragment reads for FM * FN MFMAs, which no longer divide: slot r
+// issues MFMAs [r * MFMAS / READS, (r + 1) * MFMAS / READS), three or four of them.
+// Interior tiles only (the host picks this kernel when both extents divide), one output buffer.
+// ------------------------------------------------------------------------------------------------
+template <int FM, int FN, bool KTAIL>
+__device__ __forceinline__ void gemm_rect_slabs(const GemmParams& p, char* lds, int m0, int n0, int ke, f32x4 (&acc)[FM][FN]) {
+    constexpr int BM = 32 * FM, BN = 32 * FN, BK = 64;
+    constexpr int ROWB = BK * 2, KSUB = BK / 32;
+    constexpr int UNIT_A = BM * ROWB, UNIT_W = BN * ROWB, W0 = 3 * UNIT_A;   // W ring behind the A ring
+    constexpr int PA = BM / 32, PW = BN / 32;    // buffer loads per thread per unit of A / W
+    constexpr int WROWS = 16 * FM, WCOLS = 16 * FN;
+    constexpr int READS = FM + FN, MFMAS = FM * FN;
+    constexpr int BS = READS / 4;                // slots of the last step in front of the barrier
+    constexpr int NSLOT = KSUB * READS;          // issue slots per slab
+    constexpr int GB = (KSUB - 1) * READS + BS;  // first slot behind the barrier
+    static_assert(KSUB == 2 && GB >= PA && NSLOT - GB >= PW, "schedule shape");
+    static_assert(2 * (NSLOT - GB) >= READS, "the next slab's first fragments are read two per slot behind the barrier");
+    static_assert(BM % 32 == 0 && BN % 32 == 0 && (WROWS / 2) % 8 == 0 && (WCOLS / 2) % 8 == 0, "row swizzle must not see the wave offset");
+    static_assert(3 * UNIT_A + 2 * UNIT_W <= 160 * 1024, "rings must fit the LDS");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // loader mapping as in the square kernel: LDS slot (row = pass*32 + tid/8, position tid%8) holds
+    // logical chunk position ^ ((row>>1)&7) of that row
+    const int lrow = tid >> 3;
+    const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
+    bf16_t* const base_a = const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda);
+    bf16_t* const base_b = const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw);
+    const int bytes_a = static_cast<int>(((BM - 1) * p.lda + p.K) * 2);
+    const int bytes_b = static_cast<int>(((BN - 1) * p.ldw + p.K) * 2);
+    uint32_t voff_a[PA], voff_b[PW];
+#pragma unroll
+    for (int i = 0; i < PA; ++i) voff_a[i] = static_cast<uint32_t>(((i * 32 + lrow) * p.lda + lchunk * 8) * 2);
+#pragma unroll
+    for (int i = 0; i < PW; ++i) voff_b[i] = static_cast<uint32_t>(((i * 32 + lrow) * p.ldw + lchunk * 8) * 2);
+    const int k_end = min(p.K, ke * BK);
+    auto slab_mask = [&](int kt) -> uint32_t {
+        if constexpr (KTAIL) return kt * BK + lchunk * 8 >= k_end ? kOutOfRange : 0u;
+        else return kt * BK >= k_end ? kOutOfRange : 0u;
+    };
+    auto load_a = [&](int uoff, int pass, int kt, uint32_t mask) {
+        if constexpr (KTAIL) {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_a, 0, bytes_a, kRsrcFlags), lds + uoff + pass * 4096 + wave * 1024,
+                       voff_a[pass] | mask, kt * ROWB);
+        } else {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_a, 0, mask ? 0 : bytes_a, kRsrcFlags),
+                       lds + uoff + pass * 4096 + wave * 1024, voff_a[pass], kt * ROWB);
+        }
+    };
+    auto load_w = [&](int uoff, int pass, int kt, uint32_t mask) {
+        if constexpr (KTAIL) {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_b, 0, bytes_b, kRsrcFlags), lds + W0 + uoff + pass * 4096 + wave * 1024,
+                       voff_b[pass] | mask, kt * ROWB);
+        } else {
+            load_chunk(__builtin_amdgcn_make_buffer_rsrc(base_b, 0, mask ? 0 : bytes_b, kRsrcFlags),
+                       lds + W0 + uoff + pass * 4096 + wave * 1024, voff_b[pass], kt * ROWB);
+        }
+    };
+
+    const int frow = lane & 15, fq = lane >> 4;
+    int koff_a[KSUB], koff_w[KSUB];
+#pragma unroll
+    for (int kk = 0; kk < KSUB; ++kk) {
+        const int ko = ((kk * 4 + fq) ^ ((frow >> 1) & 7)) * 16;
+        koff_a[kk] = (wm * WROWS + frow) * ROWB + ko;
+        koff_w[kk] = W0 + (wn * WCOLS + frow) * ROWB + ko;
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+
+    bf16x8 xa[2][FM], wb[2][FN];
+    auto read_frag = [&](int buf, int ua, int uw, int kk, int r) {
+        const char* pa = lds + (ua + koff_a[kk]);
+        const char* pw = lds + (uw + koff_w[kk]);
+        if (r == 0) xa[buf][0] = *reinterpret_cast<const bf16x8*>(pa);
+        else if (r <= FN) wb[buf][r - 1] = *reinterpret_cast<const bf16x8*>(pw + (r - 1) * 16 * ROWB);
+        else xa[buf][r - FN] = *reinterpret_cast<const bf16x8*>(pa + (r - FN) * 16 * ROWB);
+    };
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / FN, j = (i & 1) ? FN - 1 - idx % FN : idx % FN;   // boustrophedon, as above
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[buf][j], xa[buf][i], acc[i][j], 0, 0, 0);
+    };
+
+    // ua, ua1, ua2: units of A(kt), A(kt+1), A(kt+2); uw, uw1: of W(kt), W(kt+1); W(kt+2) takes over uw
+    // behind the barrier
+    auto slab = [&](int kt, int ua, int ua1, int ua2, int uw, int uw1, uint32_t m2, uint32_t& m3) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NSLOT; ++s) {
+            const int stp = s / READS, r = s % READS;
+            const int lo = r * MFMAS / READS, hi = (r + 1) * MFMAS / READS;
+            if (s == GB) {
+                wait_loads_and_barrier<PA>();  // W(kt+1) has landed (A(kt+1) before it); this slab's units are free
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            auto slot_reads = [&]() {
+                if (stp < KSUB - 1) {
+                    read_frag((stp & 1) ^ 1, ua, uw, stp + 1, r);
+                } else if (r >= BS) {
+                    const int f0 = 2 * (r - BS);
+                    for (int f = f0; f < f0 + 2 && f < READS; ++f) read_frag(0, ua1, uw1, 0, f);
+                }
+            };
+            if (s != 0) slot_reads();
+            mfma_one(stp & 1, lo);
+            if (s == 0) {
+                __builtin_amdgcn_sched_barrier(0);
+                slot_reads();
+            }
+            if (s == 1) m3 = slab_mask(kt + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (s < GB) {
+#pragma unroll
+                for (int i = 0; i < PA; ++i)
+                    if ((i * GB) / PA == s) load_a(ua2, i, kt + 2, m2);
+            } else if (s - GB < PW) {
+                load_w(uw, s - GB, kt + 2, m2);
+            }
+#pragma unroll
+            for (int m = lo + 1; m < hi; ++m) mfma_one(stp & 1, m);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    {
+        const uint32_t k0 = slab_mask(0), k1 = slab_mask(1);
+#pragma unroll
+        for (int i = 0; i < PA; ++i) load_a(0, i, 0, k0);
+#pragma unroll
+        for (int i = 0; i < PW; ++i) load_w(0, i, 0, k0);
+#pragma unroll
+        for (int i = 0; i < PA; ++i) load_a(UNIT_A, i, 1, k1);
+#pragma unroll
+        for (int i = 0; i < PW; ++i) load_w(UNIT_W, i, 1, k1);
+        wait_loads_and_barrier<PA + PW>();
+#pragma unroll
+        for (int r = 0; r < READS; ++r) read_frag(0, 0, 0, 0, r);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+        int ua = 0, ua1 = UNIT_A, ua2 = 2 * UNIT_A, uw = 0, uw1 = UNIT_W;
+        uint32_t m2 = slab_mask(2);
+        for (int kt = 0; kt < ke; ++kt) {
+            uint32_t m3;
+            slab(kt, ua, ua1, ua2, uw, uw1, m2, m3);
+            const int t0 = ua, t1 = uw;
+            ua = ua1; ua1 = ua2; ua2 = t0;
+            uw = uw1; uw1 = t1;
+            m2 = m3;
+        }
+    }
+    wait_vmem_all();
+    __syncthreads();
+}
+
+// Epilogue of the rectangular tile: per 16-row fragment row, bias (and GELU) in fp32, one rounding,
+// the 16 x WCOLS block parked in LDS and read back as 16-byte row segments: 16 * WCOLS / 8 of them, a
+// whole number of wave-wide accesses, lane l of access a taking segment a * 64 + l. With a gate the
+// residual rows are requested a fragment row ahead, the gate vectors once (the tile lies in one
+// batch element: the host checks).
+template <int FM, int FN, bool GELU, bool GATE>
+__device__ __forceinline__ void gemm_epilogue_rect(const GemmParams& p, f32x4 (&acc)[FM][FN], char* lds, int m0, int n0, int wave, int lane) {
+    constexpr int WROWS = 16 * FM, WCOLS = 16 * FN;
+    constexpr int C_CH = WCOLS / 8;               // 16-byte segments per row
+    constexpr int C_PITCH = WCOLS * 2 + 16;       // padded: an odd number of 16-byte units spreads the rows over the banks
+    constexpr int NACC = 16 * C_CH / 64;          // wave-wide accesses per fragment row
+    static_assert(16 * C_CH % 64 == 0, "a fragment row must be a whole number of wave-wide accesses");
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 15, fq = lane >> 4;
+    char* cw = lds + wave * (2 * 16 * C_PITCH);   // two fragment rows per wave, used in turn
+    const int wave_n0 = n0 + wn * WCOLS;
+    const int wave_m0 = m0 + wm * WROWS;
+
+    float bv[FN][4];
+    if (p.bias != nullptr) {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.bias), 0, p.N * 2, kRsrcFlags);
+#pragma unroll
+        for (int q = 0; q < FN; ++q) {
+            const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rb, (wave_n0 + q * 16 + fq * 4) * 2, 0, 0);
+            bv[q][0] = __uint_as_float(raw.x << 16);
+            bv[q][1] = __uint_as_float(raw.x & 0xffff0000u);
+            bv[q][2] = __uint_as_float(raw.y << 16);
+            bv[q][3] = __uint_as_float(raw.y & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < FN; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[q][e] = 0.0f;
+    }
+    const int waddr = frow * C_PITCH + fq * 8;    // + q * 32: column quad q of this lane's row
+    int raddr[NACC];
+    uint32_t dst_lane[NACC], res_lane[NACC];
+    Vec16<bf16_t> gt[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+        const int seg = a * 64 + lane, row = seg / C_CH, ch = seg % C_CH;
+        raddr[a] = row * C_PITCH + ch * 16;
+        dst_lane[a] = static_cast<uint32_t>(row * p.ldy * 2 + ch * 16);
+        res_lane[a] = 0;
+        if (GATE) {
+            res_lane[a] = static_cast<uint32_t>(row * p.ldresid * 2 + ch * 16);
+            gt[a] = ld16(p.gate + static_cast<int64_t>(m0 / p.rows_per_batch) * p.gate_stride + wave_n0 + ch * 8);
+        }
+    }
+    char* const dst_u = reinterpret_cast<char*>(p.Y + static_cast<int64_t>(wave_m0) * p.ldy + wave_n0);
+    const char* const res_u = GATE ? reinterpret_cast<const char*>(p.resid + static_cast<int64_t>(wave_m0) * p.ldresid + wave_n0) : nullptr;
+    Vec16<bf16_t> rs[2][NACC];
+    auto request_resid = [&](int i) {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+            rs[i & 1][a] = *reinterpret_cast<const Vec16<bf16_t>*>(res_u + static_cast<int64_t>(i) * 16 * p.ldresid * 2 + res_lane[a]);
+    };
+    if (GATE) request_resid(0);
+
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        if (GATE) {
+            if (i + 1 < FM) request_resid(i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        char* const blk = cw + (i & 1) * (16 * C_PITCH);
+#pragma unroll
+        for (int q = 0; q < FN; ++q) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = acc[i][q][e] + bv[q][e];
+                if (GELU) v[e] = tanh_gelu_fast(v[e]);
+            }
+            *reinterpret_cast<u32x2*>(blk + waddr + q * 32) = pack4_bf16(v[0], v[1], v[2], v[3]);
+        }
+        __builtin_amdgcn_wave_barrier();   // LDS operations of one wave complete in order
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(blk + raddr[a]);
+            if (GATE) {
+                const Vec16<bf16_t> r = rs[i & 1][a];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float y0 = bf2f(r.v[e]) + bf2f(f2bf(bf2f(gt[a].v[e]) * bf2f(y.v[e])));
+                    const float y1 = bf2f(r.v[e + 1]) + bf2f(f2bf(bf2f(gt[a].v[e + 1]) * bf2f(y.v[e + 1])));
+                    const uint32_t w = pack2_bf16(y0, y1);
+                    y.v[e] = static_cast<bf16_t>(w & 0xffffu);
+                    y.v[e + 1] = static_cast<bf16_t>(w >> 16);
+                }
+            }
+            *reinterpret_cast<Vec16<bf16_t>*>(dst_u + static_cast<int64_t>(i) * 16 * p.ldy * 2 + dst_lane[a]) = y;
+        }
+    }
+}
+
+template <int FM, int FN, bool KTAIL>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_rect_kernel(GemmParams p) {
+    constexpr int BM = 32 * FM, BN = 32 * FN, BK = 64;
+    __shared__ __attribute__((aligned(1024))) char lds[(3 * BM + 2 * BN) * BK * 2];
+    int tm, tn;
+    if (!tile_of_block(p, tm, tn)) return;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    f32x4 acc[FM][FN];
+    gemm_rect_slabs<FM, FN, KTAIL>(p, lds, m0, n0, (p.K + BK - 1) / BK, acc);
+    const bool gelu = p.act == FLUX_ACT_GELU_TANH;   // all columns or none: the host checks
+    if (p.gate != nullptr) {
+        if (gelu) gemm_epilogue_rect<FM, FN, true, true>(p, acc, lds, m0, n0, wave, lane);
+        else gemm_epilogue_rect<FM, FN, false, true>(p, acc, lds, m0, n0, wave, lane);
+    } else {
+        if (gelu) gemm_epilogue_rect<FM, FN, true, false>(p, acc, lds, m0, n0, wave, lane);
+        else gemm_epilogue_rect<FM, FN, false, false>(p, acc, lds, m0, n0, wave, lane);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Skinny problems (M <= 8, e.g. the Modulation projection of one conditioning vector per batch
 // element): HBM-bound on W. A wave streams the W rows of two output columns with 16-byte loads,
 // six in flight per lane, while the few activation rows come from cache; the dot products are
@@ -865,6 +1152,18 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
+constexpr int kRectFM = 9, kRectFN = 6;   // 288 x 192 tiles
+
+static void launch_rect(GemmParams& p, hipStream_t st) {
+    constexpr int BM = 32 * kRectFM, BN = 32 * kRectFN;
+    p.tiles_m = p.M / BM;
+    p.tiles_n = p.N / BN;
+    p.group_m = 4;
+    const int grid = ((p.tiles_m * p.tiles_n + 7) / 8) * 8;
+    if (p.K % 64 == 0) hipLaunchKernelGGL((gemm_nt_rect_kernel<kRectFM, kRectFN, false>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    else hipLaunchKernelGGL((gemm_nt_rect_kernel<kRectFM, kRectFN, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+}
+
 }  // namespace flux
 
 using namespace flux;
@@ -976,6 +1275,24 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
                 if (rest_tiles > 2 * kGemmCUs) break;
                 const int fill = static_cast<int>((static_cast<int64_t>(c) * tn) % kGemmCUs);
                 if ((fill == 0 || fill >= kGemmCUs * 9 / 10) && (p.gate == nullptr || (c * 256) % p.rows_per_batch == 0)) mb = c;
+            }
+        }
+        // 288 x 192 tiles when both extents divide and their rounds come out shorter than those of the
+        // square tiles (a tile is 0.84 of a square one and a little less efficient; a tail launch on
+        // 128-wide tiles costs about a third of a round): 4608 x 3072 is 216 square tiles = one round
+        // with 40 CUs idle, and 256 tiles of 288 x 192.
+        constexpr int RBM = 32 * kRectFM, RBN = 32 * kRectFN;
+        const bool rect_ok = p.M % RBM == 0 && p.N % RBN == 0 && p.vec_io && p.Y2 == nullptr &&
+                             (p.bias == nullptr || p.bias_vec) && (p.act == FLUX_ACT_NONE || p.act_begin == 0) &&
+                             (p.gate == nullptr || p.rows_per_batch % RBM == 0);
+        if (rect_ok) {
+            const double sq = mb ? static_cast<double>(static_cast<int64_t>(mb) * tn) / kGemmCUs + 0.33
+                                 : static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
+            const int64_t rt = static_cast<int64_t>(p.M / RBM) * (p.N / RBN);
+            const double rc = static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (RBM * RBN / 65536.0) * 1.04;
+            if (rc < 0.97 * sq) {
+                launch_rect(p, st);
+                return check_launch("flux_linear_bf16");
             }
         }
         if (mb == 0) {
