@@ -1028,41 +1028,77 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_rect_kernel(GemmParams p
 // folded with a wave butterfly. The kernel is instantiated per row count, so it has no row tests.
 // ------------------------------------------------------------------------------------------------
 constexpr int kGemvCols = 2;  // output columns per wave
+constexpr int kGemvSiluLds = 48 * 1024;  // bytes of LDS for the (activated) input rows (bf16)
+// 16-byte vectors of a W row a lane requests at once: a whole row of 3072 for one or two activation rows,
+// half of that when more rows' products need the registers
+constexpr int gemv_depth(int rows) { return rows <= 2 ? 6 : 3; }
 
-template <int MM>
+// SILU_LDS: the few activation rows are staged in LDS once per workgroup, with the input activation
+// x * sigmoid(x) applied on the way (rounded to bf16, as the separate operator would leave it). Every
+// wave needs all K values of every row: read from memory inside the K loop they queue behind the W
+// loads of the wave (the memory counter is in-order), and the activation, two transcendentals per
+// value, would be repeated by each of the N / 2 waves. Rows that do not fit the LDS budget are read
+// from memory as they are needed.
+// EXACT: K = 512 * U, so every lane has exactly U vectors per row and the K loop runs once, without tests.
+template <int MM, bool SILU_LDS, bool EXACT>
 __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
-    constexpr int CPW = kGemvCols, U = 3;  // CPW * U 16-byte loads of W in flight per lane
+    constexpr int CPW = kGemvCols, U = gemv_depth(MM);  // CPW * U 16-byte loads of W in flight per lane: a whole row of 3072
+    extern __shared__ __attribute__((aligned(16))) char act_lds[];
     const int lane = threadIdx.x & 63;
     const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CPW;
-    if (n0 >= p.N) return;  // whole wave leaves together
-    float acc[CPW][MM];
-#pragma unroll
-    for (int c = 0; c < CPW; ++c)
-#pragma unroll
-        for (int m = 0; m < MM; ++m) acc[c][m] = 0.0f;
     const bf16_t* wrow[CPW];
 #pragma unroll
-    for (int c = 0; c < CPW; ++c) wrow[c] = p.W + static_cast<int64_t>(n0 + c < p.N ? n0 + c : n0) * p.ldw;
-    for (int k0 = lane * 8; k0 < p.K; k0 += 512 * U) {
-        Vec16<bf16_t> w[U][CPW];
+    for (int c = 0; c < CPW; ++c) wrow[c] = p.W + static_cast<int64_t>(n0 + c < p.N ? n0 + c : (n0 < p.N ? n0 : p.N - 1)) * p.ldw;
+    // the first group of W loads goes out before the activation is worked on
+    Vec16<bf16_t> w[U][CPW];
+    auto request_w = [&](int k0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int k = k0 + u * 512;
             // past the end: a harmless re-read, skipped below
 #pragma unroll
-            for (int c = 0; c < CPW; ++c) w[u][c] = ld16(wrow[c] + (k < p.K ? k : k0));
+            for (int c = 0; c < CPW; ++c) w[u][c] = ld16(wrow[c] + (EXACT || k < p.K ? k : k0));
         }
+    };
+    if (EXACT || lane * 8 < p.K) request_w(lane * 8);
+    if (SILU_LDS) {
+        bf16_t* dst = reinterpret_cast<bf16_t*>(act_lds);
+        for (int i = threadIdx.x * 8; i < MM * p.K; i += 256 * 8) {   // K is a multiple of 8: a vector stays inside one row
+            const int m = i / p.K, k = i - m * p.K;
+            const Vec16<bf16_t> a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
+            Vec16<bf16_t> o = a;
+            if (p.in_silu) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = bf2f(a.v[e]);
+                    o.v[e] = f2bf(f * __builtin_amdgcn_rcpf(1.0f + __expf(-f)));
+                }
+            }
+            *reinterpret_cast<Vec16<bf16_t>*>(dst + i) = o;
+        }
+        __syncthreads();
+    }
+    if (n0 >= p.N) return;  // whole wave leaves together (after the barrier)
+    float acc[CPW][MM];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+        for (int m = 0; m < MM; ++m) acc[c][m] = 0.0f;
+    for (int k0 = lane * 8; k0 < (EXACT ? 512 : p.K); k0 += 512 * U) {
+        if (!EXACT && k0 != lane * 8) request_w(k0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int k = k0 + u * 512;
-            if (k >= p.K) break;
+            if (!EXACT && k >= p.K) break;
             float af[MM][8];
 #pragma unroll
             for (int m = 0; m < MM; ++m) {
-                const Vec16<bf16_t> a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
+                Vec16<bf16_t> a;
+                if (SILU_LDS) a = *reinterpret_cast<const Vec16<bf16_t>*>(act_lds + (static_cast<size_t>(m) * p.K + k) * 2);
+                else a = ld16(p.A + static_cast<int64_t>(m) * p.lda + k);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) af[m][e] = bf2f(a.v[e]);
-                if (p.in_silu) {
+                if (!SILU_LDS && p.in_silu) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) af[m][e] = bf2f(f2bf(af[m][e] * __builtin_amdgcn_rcpf(1.0f + __expf(-af[m][e]))));
                 }
@@ -1108,7 +1144,12 @@ __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
 template <int MM>
 static void launch_gemv(const GemmParams& p, hipStream_t st) {
     const unsigned grid = (unsigned)((p.N + 4 * kGemvCols - 1) / (4 * kGemvCols));
-    hipLaunchKernelGGL((gemv_small_m_kernel<MM>), dim3(grid), dim3(256), 0, st, p);
+    const size_t act_bytes = static_cast<size_t>(MM) * p.K * 2;
+    const bool lds = act_bytes <= kGemvSiluLds, exact = p.K == 512 * gemv_depth(MM);
+    if (lds && exact) hipLaunchKernelGGL((gemv_small_m_kernel<MM, true, true>), dim3(grid), dim3(256), act_bytes, st, p);
+    else if (lds) hipLaunchKernelGGL((gemv_small_m_kernel<MM, true, false>), dim3(grid), dim3(256), act_bytes, st, p);
+    else if (exact) hipLaunchKernelGGL((gemv_small_m_kernel<MM, false, true>), dim3(grid), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gemv_small_m_kernel<MM, false, false>), dim3(grid), dim3(256), 0, st, p);
 }
 
 // ------------------------------------------------------------------------------------------------
