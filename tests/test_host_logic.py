@@ -98,6 +98,18 @@ def test_state_dicts_are_interchangeable():
     assert isinstance(modules.MLP(8, 32)[1], torch.nn.Identity)
 
 
+def test_linear_launch_metadata_matches_the_reference_hook():
+    """kernels/linear.py:9-19 of the reference: name with the problem size, flops16 = 2 M N K, bytes = A + W + C."""
+    import sys
+    import triton_kernels.kernels.linear  # noqa: F401  (the package re-exports the function under the same name)
+    lin = sys.modules["triton_kernels.kernels.linear"]
+    md = lin.linear_launch_metadata(4608, 21504, 3072)
+    assert md["name"].endswith("[M=4608, N=21504, K=3072]")
+    assert md["flops16"] == 2.0 * 4608 * 21504 * 3072
+    assert md["bytes"] == 2 * (4608 * 3072 + 21504 * 3072 + 4608 * 21504)
+    assert lin.launch_hook is None
+
+
 def test_hip_op_launch_spelling():
     calls = []
     op = HipOp(lambda a, b, scale=1: calls.append((a, b, scale)) or "ok", "demo")

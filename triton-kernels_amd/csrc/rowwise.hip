@@ -62,13 +62,25 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_regs(
     const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / G;
     const bool row_ok = row < rows;
 
+    // Offset of the row in the strided [d0, d1, d2] view. The host merges dimensions whose strides
+    // allow it, so an evenly strided tensor arrives as d1 = 1 and needs no division; other views
+    // divide in 32 bits when the row count allows (a 64-bit division costs a hundred instructions,
+    // which at one vector per lane is more than the rest of the kernel).
     int64_t off = 0;
     if (row_ok) {
-        int64_t i2 = row % d2;
-        int64_t t = row / d2;
-        int64_t i1 = t % d1;
-        int64_t i0 = t / d1;
-        off = i0 * s0 + i1 * s1 + i2 * s2;
+        if (d1 == 1 && row < d2) {
+            off = row * s2;
+        } else if (rows <= 0x7fffffffLL) {
+            const uint32_t r32 = static_cast<uint32_t>(row), e2 = static_cast<uint32_t>(d2), e1 = static_cast<uint32_t>(d1);
+            const uint32_t t = r32 / e2, i2 = r32 - t * e2, i0 = t / e1, i1 = t - i0 * e1;
+            off = i0 * s0 + i1 * s1 + static_cast<int64_t>(i2) * s2;
+        } else {
+            int64_t i2 = row % d2;
+            int64_t t = row / d2;
+            int64_t i1 = t % d1;
+            int64_t i0 = t / d1;
+            off = i0 * s0 + i1 * s1 + i2 * s2;
+        }
     }
     RowRegs<T, G, ITER> r;
     r.load(x + off, lane, n, row_ok);
@@ -413,6 +425,9 @@ static int rms_fwd_launch(const void* x, const void* scale, void* y, float* rstd
     RowPlan plan = plan_row(n, VEC);
     const bool vec_ok = aligned16(x) && aligned16(y) && s0 % VEC == 0 && s1 % VEC == 0 && s2 % VEC == 0 &&
                         (sizeof(TS) * VEC != 16 || aligned16(scale));
+    // merge dimensions that are evenly strided: [d0, d1, d2] -> [1, 1, rows] for a contiguous tensor
+    if (d0 == 1 || s0 == d1 * s1) { d1 *= d0; d0 = 1; }
+    if (d0 == 1 && (d1 == 1 || s1 == d2 * s2)) { d2 *= d1; d1 = 1; }
     if (plan.G != 0 && vec_ok) {
 #define CALL(G_, I_)                                                                                          \
     hipLaunchKernelGGL((rms_norm_fwd_regs<T, TS, G_, I_>), dim3((unsigned)((rows + kBlock / G_ - 1) / (kBlock / G_))), \

@@ -14,6 +14,19 @@ _ACTIVATIONS = {"": nv.ACT_NONE, "GELU": nv.ACT_GELU_TANH}
 _PLANS = {torch.bfloat16: {"tile": (256, 256, 64), "waves": 4, "mfma": "16x16x32"}}
 
 
+# Optional callable(dict) invoked with the metadata of every launch of the linear kernel, on the launching
+# thread, right before the launch. Profilers and benchmarks set it (e.g. to open a named range); None
+# costs nothing. The dictionary is what the reference attaches to its launches for its profiler
+# (kernels/linear.py:9-19): "name" with the problem size, "flops16" = 2 M N K and "bytes" = the three
+# matrices once.
+launch_hook = None
+
+
+def linear_launch_metadata(M: int, N: int, K: int, elem_bytes: int = 2, epilogue: str = "") -> dict:
+    name = f"flux_linear_bf16 [M={M}, N={N}, K={K}]" + (f" {epilogue}" if epilogue else "")
+    return {"name": name, f"flops{elem_bytes * 8}": 2.0 * M * N * K, "bytes": elem_bytes * (M * K + N * K + M * N)}
+
+
 def _rows_2d(x: Tensor, K: int) -> Tensor:
     x2 = x.reshape(-1, K)
     if x2.shape[0] > 1 and (x2.stride(1) != 1 or x2.stride(0) < K):
@@ -101,6 +114,10 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
         f.eps = float(qk.get("eps", 1e-6))
         a.qk = ctypes.pointer(f)
         keep = (f, qs, ks, pe2)
+    if launch_hook is not None:
+        parts = [activation and f"{activation}>={act_begin}", split is not None and f"split@{split}", gate is not None and "gated-residual",
+                 qk is not None and "qk-norm-rope", in_activation and f"in:{in_activation}"]
+        launch_hook(linear_launch_metadata(M, N, K, x.element_size(), "+".join(p for p in parts if p)))
     with nv.on_device(dev):
         rc = nv.lib().flux_linear_bf16(nv.byref(a), nv.stream_ptr(dev))
     nv.check(rc, "flux_linear_bf16")
