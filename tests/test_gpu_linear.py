@@ -167,7 +167,11 @@ def test_linear_gated_residual_epilogue(B, L, hid, K):
 
 
 @pytest.mark.parametrize("B,L,H,mlp,bias,per_batch_pe", [(2, 256, 3, 1152, True, False), (1, 512, 2, 256, False, False),
-                                                         (2, 256, 2, 256, True, True), (1, 4608, 24, 12288, True, False)])
+                                                         (2, 256, 2, 256, True, True), (1, 4608, 24, 12288, True, False),
+                                                         # ragged: rows and sequence length no multiple of the tile, tiles that
+                                                         # hold the end of one batch element and the start of the next
+                                                         (3, 300, 2, 256, True, True), (2, 421, 3, 1152, False, False),
+                                                         (1, 333, 2, 256, True, False), (3, 4336, 24, 12288, True, False)])
 def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
     """linear1 with QKNorm + RoPE in the epilogue: q and k leave as [B,H,L,128], v and the GELU'd mlp
     columns as in the split epilogue. Checked against the oracle chain on the un-fused projection
@@ -186,7 +190,7 @@ def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
     both = torch.zeros(M, hid + mlp, dtype=torch.bfloat16, device=DEV)
     q = torch.empty(B, H, L, D, dtype=torch.bfloat16, device=DEV)
     k = torch.empty_like(q)
-    assert qk_fusable(x, w, L, D) == ((M // 256) * (N // 256) >= 160)   # small ones are taken, just not preferred
+    assert qk_fusable(x, w, L, D) == (-(-M // 256) * (N // 256) >= 160)   # small ones are taken, just not preferred
     tk.linear_into(x, w, b, activation="GELU", act_begin=3 * hid, out=qkv, out2=both[:, hid:], split=3 * hid,
                    qk=dict(q_out=q, k_out=k, q_scale=qs, k_scale=ks, pe=pe, heads=H, seq_len=L, eps=1e-6))
 
@@ -199,14 +203,25 @@ def test_linear_qk_norm_rope_epilogue(B, L, H, mlp, bias, per_batch_pe):
     assert (qkv[:, :2 * hid] == 0).all()                               # q and k columns are not written
     heads = qkv_u.view(B, L, 3, H, D).permute(2, 0, 3, 1, 4)
     q_u, k_u, _ = tk.qkv_prep(heads[0], heads[1], None, pe=pe, q_scale_img=qs, k_scale_img=ks)
-    torch.testing.assert_close(q, q_u, atol=1e-2, rtol=1e-2)
-    torch.testing.assert_close(k, k_u, atol=1e-2, rtol=1e-2)
     # oracle chain on the bf16 projection
     qn = oracle.rms_norm_ref(heads[0].cpu(), qs.cpu())
     kn = oracle.rms_norm_ref(heads[1].cpu(), ks.cpu())
     rq, rk = oracle.apply_rope_ref(qn, kn, pe.cpu())
-    torch.testing.assert_close(q.cpu(), rq, atol=2e-2, rtol=2e-2)
-    torch.testing.assert_close(k.cpu(), rk, atol=2e-2, rtol=2e-2)
+
+    def close(got, want, normed, atol, rtol):
+        """atol + rtol |want|, plus what one bf16 ulp of a normalised value is worth behind the 2 x 2 matrix:
+        where x * rstd falls on a rounding boundary two correct evaluations may round it either way, and
+        the table here is random (entries of several units, rows that cancel), which magnifies that ulp."""
+        xn = normed.float().reshape(*normed.shape[:-1], -1, 1, 2).abs()
+        amp = (pe.cpu().float().abs() * xn).sum(-1).reshape(normed.shape)
+        err = (got.cpu().float() - want.cpu().float()).abs()
+        assert (err <= atol + rtol * want.cpu().float().abs() + 2.0 ** -7 * amp).all(), err.max().item()
+        assert err.mean().item() < 2e-3
+
+    close(q, q_u, qn, 1e-2, 1e-2)
+    close(k, k_u, kn, 1e-2, 1e-2)
+    close(q, rq, qn, 2e-2, 2e-2)
+    close(k, rk, kn, 2e-2, 2e-2)
 
 
 @pytest.mark.parametrize("M", [1, 2, 5, 8])

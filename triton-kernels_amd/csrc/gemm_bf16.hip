@@ -341,8 +341,13 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, f32x4 (&
 // (the projection's output), RMS-normalised over the head (x * rstd rounded, times scale rounded),
 // rotated by the 2x2 matrices of its position and written to [B, heads, out_len, 128]. A lane holds
 // 32 of a row's 128 columns; the other 96 are in the lanes 16, 32 and 48 further on, so the sum of
-// squares takes two cross-lane steps. Interior tiles only; a tile lies inside one batch element.
-template <int MI, int NJ>
+// squares takes two cross-lane steps. RAGGED = false: the tile is interior and lies inside one batch
+// element, so its rows are consecutive positions of one (batch, head). RAGGED = true: the tile may run
+// past the last row and may hold the last rows of one batch element followed by the first of the next
+// (at most one such boundary: sequences are at least a tile long); rows past the end are computed on
+// clamped table rows and not stored, rows behind the boundary take their table rows and their
+// destination from the next batch element.
+template <int MI, int NJ, bool RAGGED>
 __device__ __forceinline__ void gemm_epilogue_qk(const GemmParams& p, f32x4 (&acc)[2 * MI][2 * NJ], char* lds, int m0, int n0,
                                                  int wave, int lane) {
     constexpr int WROWS = 32 * MI, WCOLS = 32 * NJ;
@@ -396,6 +401,13 @@ __device__ __forceinline__ void gemm_epilogue_qk(const GemmParams& p, f32x4 (&ac
     }
     // rotation table of this lane's columns: 8 floats per quad, row stride 2 * 128 floats
     const float* pe_lane = p.pe + static_cast<int64_t>(batch) * p.pe_batch_stride + static_cast<int64_t>(pos_w + frow) * (2 * WCOLS) + fq * 8;
+    // RAGGED: rows of the wave's sub-tile from `boundary` on belong to the next batch element, whose
+    // positions restart: their table row is pe_next floats and their output row out_next bytes further on
+    const int boundary = RAGGED ? (batch + 1) * p.qk_seq_len - wave_m0 : WROWS;
+    const int64_t pe_next = RAGGED ? p.pe_batch_stride - static_cast<int64_t>(p.qk_seq_len) * (2 * WCOLS) : 0;
+    const uint32_t out_next = RAGGED ? static_cast<uint32_t>((static_cast<int64_t>(p.qk_heads) * p.qk_out_len - p.qk_seq_len) * (WCOLS * 2)) : 0u;
+    const int rows_valid = RAGGED ? p.M - wave_m0 : WROWS;   // rows of the sub-tile inside the matrix
+    if (RAGGED && rows_valid <= 0) return;                   // nothing of this wave's to store (no workgroup barrier follows)
     char* dst_u = reinterpret_cast<char*>((is_k ? p.k_out : p.q_out) +
                                           ((static_cast<int64_t>(batch) * p.qk_heads + head) * p.qk_out_len + pos_w) * WCOLS);
     const uint32_t dst_lane = static_cast<uint32_t>(rrow * (WCOLS * 2) + rch * 16);
@@ -411,6 +423,10 @@ __device__ __forceinline__ void gemm_epilogue_qk(const GemmParams& p, f32x4 (&ac
             f32x4 fr[NQ][2];
             {
                 const float* pr = pe_lane + (i * 32 + t * 16) * (2 * WCOLS);
+                if (RAGGED) {
+                    const int r = min(i * 32 + t * 16 + frow, rows_valid - 1);   // past the end: the last valid row's entries
+                    pr = pe_lane + static_cast<int64_t>(r - frow) * (2 * WCOLS) + (r >= boundary ? pe_next : 0);
+                }
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     fr[q][0] = *reinterpret_cast<const f32x4*>(pr + q * 32);
@@ -461,7 +477,13 @@ __device__ __forceinline__ void gemm_epilogue_qk(const GemmParams& p, f32x4 (&ac
         for (int it = 0; it < NIT; ++it) {
             const int row_u = i * 32 + it * RPI;
             const Vec16<bf16_t> y = *reinterpret_cast<const Vec16<bf16_t>*>(cw + (i * 32 + (it / NSW) * NSW * RPI) * C_PITCH + raddr[it % NSW]);
-            *reinterpret_cast<Vec16<bf16_t>*>(dst_u + static_cast<int64_t>(row_u) * (WCOLS * 2) + dst_lane) = y;
+            if (RAGGED) {
+                const int r = row_u + rrow;
+                if (r < rows_valid)
+                    *reinterpret_cast<Vec16<bf16_t>*>(dst_u + static_cast<int64_t>(row_u) * (WCOLS * 2) + (dst_lane + (r >= boundary ? out_next : 0u))) = y;
+            } else {
+                *reinterpret_cast<Vec16<bf16_t>*>(dst_u + static_cast<int64_t>(row_u) * (WCOLS * 2) + dst_lane) = y;
+            }
         }
     }
 }
@@ -474,8 +496,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x4 (&acc)[
     const bool gelu_all = p.act == FLUX_ACT_GELU_TANH && wave_n0 >= p.act_begin;
     const bool gelu_none = p.act != FLUX_ACT_GELU_TANH || wave_n0 + WCOLS <= p.act_begin;
     if constexpr (NJ == 4) {
-        if (wave_n0 < p.qk_cols) {   // the host admits the fusion only when every such tile is interior
-            gemm_epilogue_qk<MI, NJ>(p, acc, lds, m0, n0, wave, lane);
+        if (wave_n0 < p.qk_cols) {   // the host admits the fusion only when the q/k columns are whole tiles
+            const bool ragged = m0 + BM > p.M || m0 / p.qk_seq_len != (m0 + BM - 1) / p.qk_seq_len;
+            if (ragged) gemm_epilogue_qk<MI, NJ, true>(p, acc, lds, m0, n0, wave, lane);
+            else gemm_epilogue_qk<MI, NJ, false>(p, acc, lds, m0, n0, wave, lane);
             return;
         }
     }
@@ -1249,8 +1273,9 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
         const flux_linear_qk_fusion* f = a->qk;
         if (!f->q_out || !f->k_out || !f->q_scale || !f->k_scale || !f->pe) return fail(FLUX_E_NULL, "flux_linear_bf16: qk fusion with a null pointer");
         const int64_t cols = 2 * f->heads * 128;
-        const bool shape_ok = f->heads > 0 && f->seq_len > 0 && f->seq_len % 256 == 0 && a->M % f->seq_len == 0 && a->N % 256 == 0 &&
+        const bool shape_ok = f->heads > 0 && f->seq_len >= 256 && a->M % f->seq_len == 0 && a->N % 256 == 0 &&
                               cols <= a->N && f->pos0 >= 0 && f->pos0 + f->seq_len <= f->out_len && f->out_len < 0x7fffff &&
+                              f->heads * f->out_len * 256 < 0x7fffffffLL &&
                               f->pe_batch_stride >= 0 && a->K > 0 && a->K % 8 == 0;
         const bool epi_ok = a->gate == nullptr && p.act_begin >= cols && p.split_n >= cols &&
                             (a->bias == nullptr || p.bias_vec) && p.vec_io;
@@ -1259,8 +1284,8 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
                             aligned16(a->A) && aligned16(a->W) && a->lda % 8 == 0 && a->ldw % 8 == 0 &&
                             a->lda * 2 * 256 < 0x7fffffffLL && a->ldw * 2 * 256 < 0x7fffffffLL;
         if (!shape_ok || !epi_ok || !ptr_ok)
-            return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: qk fusion needs M, N and seq_len in multiples of 256, aligned operands, "
-                                            "no gate, and GELU / split columns behind the k heads");
+            return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: qk fusion needs N in multiples of 256, sequences of at least 256 rows, "
+                                            "aligned operands, no gate, and GELU / split columns behind the k heads");
         p.q_out = static_cast<bf16_t*>(f->q_out); p.k_out = static_cast<bf16_t*>(f->k_out);
         p.q_scale = static_cast<const bf16_t*>(f->q_scale); p.k_scale = static_cast<const bf16_t*>(f->k_scale);
         p.pe = f->pe; p.pe_batch_stride = f->pe_batch_stride;

@@ -127,13 +127,13 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
 
 def qk_fusable(x: Tensor, w: Tensor, seq_len: int, head_dim: int) -> bool:
     """Whether linear_into(..., qk=...) takes this projection and is worth it: bf16, heads of 128,
-    rows, columns and sequence length in multiples of the 256-wide tile (so every q/k tile is
-    interior and lies inside one batch element), and enough of those tiles that the library would
-    pick them anyway (the fused epilogue exists for the 256-wide tile only)."""
+    columns in multiples of the 256-wide tile, sequences of at least one tile (a tile then holds rows
+    of at most two batch elements; ragged row counts and sequence lengths are fine), and enough
+    tiles that the library would pick the 256-wide ones anyway (the fused epilogue exists for them only)."""
     M = x.numel() // x.shape[-1]
     N = w.shape[0]
-    return (x.dtype == torch.bfloat16 and head_dim == 128 and seq_len > 0 and seq_len % 256 == 0 and M % seq_len == 0
-            and N % 256 == 0 and w.shape[1] % 8 == 0 and (M // 256) * (N // 256) >= 160)
+    return (x.dtype == torch.bfloat16 and head_dim == 128 and seq_len >= 256 and M % seq_len == 0
+            and N % 256 == 0 and w.shape[1] % 8 == 0 and -(-M // 256) * (N // 256) >= 160)
 
 
 def linear(x: Tensor, w: Tensor, b: Tensor | None, activation: str = "") -> Tensor:

@@ -160,8 +160,8 @@ class SingleStreamBlock(nn.Module):
     """DiT block with parallel attention and MLP branches (https://arxiv.org/abs/2302.05442)."""
 
     fused = True
-    # QKNorm + RoPE inside linear1's epilogue when the shapes allow (heads of 128, sequence length a
-    # multiple of 256); otherwise, or with this switched off, one preparation kernel behind linear1
+    # QKNorm + RoPE inside linear1's epilogue when the shapes allow (heads of 128, sequences of at least
+    # 256 tokens); otherwise, or with this switched off, one preparation kernel behind linear1
     fuse_qk_epilogue = True
     # Optional callable(stage, edge), invoked on the launching thread right before (edge "begin") and
     # right after ("end") the launch of a stage of the forward: "modulation", "layer_norm" and, in the
