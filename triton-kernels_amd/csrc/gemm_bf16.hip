@@ -1350,7 +1350,8 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
         constexpr int RBM = 32 * kRectFM, RBN = 32 * kRectFN;
         const bool rect_ok = p.M % RBM == 0 && p.N % RBN == 0 && p.vec_io && p.Y2 == nullptr &&
                              (p.bias == nullptr || p.bias_vec) && (p.act == FLUX_ACT_NONE || p.act_begin == 0) &&
-                             (p.gate == nullptr || p.rows_per_batch % RBM == 0);
+                             (p.gate == nullptr || p.rows_per_batch % RBM == 0) &&
+                             a->lda * 2 * RBM < 0x7fffffffLL && a->ldw * 2 * RBN < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
         if (rect_ok) {
             const double sq = mb ? static_cast<double>(static_cast<int64_t>(mb) * tn) / kGemmCUs + 0.33
                                  : static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
