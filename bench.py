@@ -254,7 +254,7 @@ def kernel_cases(torch, extra=False):
                 x, _ = cfg.config1(dev)
                 keep, launches = [], []
                 for _ in range(n_sets(mult * 2 * qk_elems * 2)):
-                    q_ = x.expand(mult, -1, -1, -1).contiguous()
+                    q_ = x.expand(mult, -1, -1, -1).clone(memory_format=torch.contiguous_format)   # a buffer of its own per set
                     oq = torch.empty_like(q_)
                     a = prep_args(None, None, None, None, q_, None, None, oq, None, None, False, 0, batch=mult)
                     keep.append((q_, oq, a))
