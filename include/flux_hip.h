@@ -147,9 +147,11 @@ int flux_qkv_prep(const flux_qkv_prep_args* args, void* stream);
  * (x * rsqrt(mean x^2 + eps) rounded, times scale rounded), rotated with the 2x2 matrices of its
  * position (pe[pos][c/2] = [[f00,f01],[f10,f11]] for the column pair c, c+1) and stored at
  * q_out / k_out [b, head, pos0 + l, :], where row m of the product is (b, l) = (m / seq_len,
- * m % seq_len). They are not written to Y. Requirements (else FLUX_E_UNSUPPORTED): M and seq_len
- * multiples of 256, N a multiple of 256, 16-byte aligned pointers, no gate, act_begin and split_n
- * at or past 2*heads*128, K a multiple of 8. */
+ * m % seq_len). They are not written to Y. Any row count M = B * seq_len is taken: tiles that run
+ * past the last row, or that hold the last rows of one batch element and the first of the next,
+ * take a checked form of the epilogue. Requirements (else FLUX_E_UNSUPPORTED): seq_len >= 256,
+ * N a multiple of 256, 16-byte aligned pointers, no gate, act_begin and split_n at or past
+ * 2*heads*128, K a multiple of 8. */
 typedef struct flux_linear_qk_fusion {
     void* q_out; void* k_out;                  /* [B, heads, out_len, 128] bf16, contiguous */
     const void* q_scale; const void* k_scale;  /* [128] bf16 */
