@@ -32,13 +32,23 @@ __device__ __forceinline__ bf16_t f2bf(float f) {
     return __builtin_bit_cast(bf16_t, b);
 }
 
+// fp32 -> nearest bf16 -> fp32 in one instruction: the convert packs two values into the halves of a
+// register, and a value placed in the high half over a zero low half is already the fp32 bit
+// pattern of its rounded self (v_cvt_pk_bf16_f32 dst, 0, f), so no shift follows.
+__device__ __forceinline__ float round_bf16(float f) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {0.0f, f};
+    return __uint_as_float(__builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t)));
+}
+
 // Rounds through the storage type: identity for fp32, bf16 round trip for bf16.
 template <typename T> struct Elem;
 template <> struct Elem<bf16_t> {
     static constexpr int VEC = 8;  // elements per 16-byte access
     static __device__ __forceinline__ float load(bf16_t v) { return bf2f(v); }
     static __device__ __forceinline__ bf16_t store(float f) { return f2bf(f); }
-    static __device__ __forceinline__ float round(float f) { return bf2f(f2bf(f)); }
+    static __device__ __forceinline__ float round(float f) { return round_bf16(f); }
 };
 template <> struct Elem<float> {
     static constexpr int VEC = 4;

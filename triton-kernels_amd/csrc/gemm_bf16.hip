@@ -1124,7 +1124,7 @@ __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
                 for (int e = 0; e < 8; ++e) af[m][e] = bf2f(a.v[e]);
                 if (!SILU_LDS && p.in_silu) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) af[m][e] = bf2f(f2bf(af[m][e] * __builtin_amdgcn_rcpf(1.0f + __expf(-af[m][e]))));
+                    for (int e = 0; e < 8; ++e) af[m][e] = round_bf16(af[m][e] * __builtin_amdgcn_rcpf(1.0f + __expf(-af[m][e])));
                 }
             }
 #pragma unroll
@@ -1151,11 +1151,11 @@ __global__ __launch_bounds__(256) void gemv_small_m_kernel(GemmParams p) {
             for (int m = 0; m < MM; ++m) {
                 float t = acc[c][m] + b;
                 if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
-                t = bf2f(f2bf(t));
+                t = round_bf16(t);
                 if (p.gate != nullptr) {
                     const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
                     const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
-                    t = r + bf2f(f2bf(g * t));
+                    t = r + round_bf16(g * t);
                 }
                 bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
                                             : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
@@ -1189,16 +1189,16 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmParams p) {
     float acc = 0.0f;
     for (int k = 0; k < p.K; ++k) {
         float x = bf2f(a[k]);
-        if (p.in_silu) x = bf2f(f2bf(x * __builtin_amdgcn_rcpf(1.0f + __expf(-x))));
+        if (p.in_silu) x = round_bf16(x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)));
         acc += x * bf2f(w[k]);
     }
     float t = acc + (p.bias ? bf2f(p.bias[n]) : 0.0f);
     if (p.act == FLUX_ACT_GELU_TANH && n >= p.act_begin) t = gelu_tanh_f32(t);
-    t = bf2f(f2bf(t));
+    t = round_bf16(t);
     if (p.gate != nullptr) {
         const float g = bf2f(p.gate[static_cast<int64_t>(m / p.rows_per_batch) * p.gate_stride + n]);
         const float r = bf2f(p.resid[static_cast<int64_t>(m) * p.ldresid + n]);
-        t = r + bf2f(f2bf(g * t));
+        t = r + round_bf16(g * t);
     }
     bf16_t* dst = n < p.split_n ? p.Y + static_cast<int64_t>(m) * p.ldy + n
                                 : p.Y2 + static_cast<int64_t>(m) * p.ldy2 + (n - p.split_n + p.y2_col0);
