@@ -1344,19 +1344,25 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
             }
         }
         // 288 x 192 tiles when both extents divide and their rounds come out shorter than those of the
-        // square tiles (a tile is 0.84 of a square one and a little less efficient; a tail launch on
-        // 128-wide tiles costs about a third of a round): 4608 x 3072 is 216 square tiles = one round
-        // with 40 CUs idle, and 256 tiles of 288 x 192.
+        // square tiles. Measured at K = 3072: a round of square tiles 69 us, a round of 288 x 192 tiles
+        // 62 us (0.84 of the work at 1.06 times the cost per flop), a tail launch on 128-wide tiles
+        // 0.65 of a square round per wave of 512 workgroups plus a kernel boundary. 4608 x 3072 is
+        // 216 square tiles = one round with 40 CUs idle, and 256 tiles of 288 x 192; 4608 x 12288 is
+        // 3 square rounds and a tail, or 4 rounds of 288 x 192.
         constexpr int RBM = 32 * kRectFM, RBN = 32 * kRectFN;
         const bool rect_ok = p.M % RBM == 0 && p.N % RBN == 0 && p.vec_io && p.Y2 == nullptr &&
                              (p.bias == nullptr || p.bias_vec) && (p.act == FLUX_ACT_NONE || p.act_begin == 0) &&
                              (p.gate == nullptr || p.rows_per_batch % RBM == 0) &&
                              a->lda * 2 * RBM < 0x7fffffffLL && a->ldw * 2 * RBN < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
         if (rect_ok) {
-            const double sq = mb ? static_cast<double>(static_cast<int64_t>(mb) * tn) / kGemmCUs + 0.33
-                                 : static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
+            double sq = static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
+            if (mb) {
+                const int64_t rest_tiles = ((p.M - static_cast<int64_t>(mb) * 256 + 127) / 128) * ((p.N + 127) / 128);
+                sq = static_cast<double>((static_cast<int64_t>(mb) * tn + kGemmCUs - 1) / kGemmCUs) +
+                     0.65 * static_cast<double>((rest_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)) + 0.1;
+            }
             const int64_t rt = static_cast<int64_t>(p.M / RBM) * (p.N / RBN);
-            const double rc = static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (RBM * RBN / 65536.0) * 1.04;
+            const double rc = static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (RBM * RBN / 65536.0) * 1.06;
             if (rc < 0.97 * sq) {
                 launch_rect(p, st);
                 return check_launch("flux_linear_bf16");
