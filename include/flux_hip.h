@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FLUX_ABI_VERSION 3
+#define FLUX_ABI_VERSION 4
 
 enum flux_dtype { FLUX_BF16 = 0, FLUX_F32 = 1 };
 
@@ -171,7 +171,14 @@ typedef struct flux_linear_args {
     int64_t ldresid, gate_batch_stride, rows_per_batch;
     int32_t act; int32_t in_act; int64_t act_begin;
     const flux_linear_qk_fusion* qk;           /* null = off */
+    int64_t flags;                             /* FLUX_LINEAR_* bits, 0 = none */
 } flux_linear_args;
+
+/* flags: the launch will run beside work of another stream (the txt chain beside the img chain of
+ * the double-stream block). The library then keeps the tile shape whose last round leaves CUs free
+ * for that work instead of the one that fills every round of the 256 CUs exactly, which is the
+ * faster one only when the launch has the GPU to itself. The result is the same bits either way. */
+#define FLUX_LINEAR_SHARED_GPU 1
 
 int flux_linear_bf16(const flux_linear_args* args, void* stream);
 

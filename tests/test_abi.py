@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in flux_hip.h but not exported"
     assert set(names) == set(nv.SIGNATURES), "ctypes binding table and header disagree"
-    assert nv.lib().flux_abi_version() == 3
+    assert nv.lib().flux_abi_version() == 4
 
 
 def test_struct_layouts_match_the_header(tmp_path):
@@ -78,6 +78,10 @@ def test_argument_checks_reject_before_launch():
     assert lib.flux_linear_bf16(ctypes.byref(la), None) == -6                                           # fused SiLU on more than 8 rows
     assert b"M <= 8" in lib.flux_last_error()
     la.in_act, la.M = 0, 4
+    la.flags = 2
+    assert lib.flux_linear_bf16(ctypes.byref(la), None) == -6                                           # unknown flag bit
+    assert b"flags" in lib.flux_last_error()
+    la.flags = nv.LINEAR_SHARED_GPU
     qf = nv.LinearQKFusion()
     qf.q_out = qf.k_out = qf.q_scale = qf.k_scale = qf.pe = p
     qf.heads, qf.seq_len, qf.out_len = 1, 256, 256

@@ -78,9 +78,14 @@ def test_linear_ragged_shapes(M, N, K, bias):
     (1, 2304, 6144, 136, "GELU", True, False),  # GELU on every column
     (1, 2304, 6144, 64, "", True, False),       # a single slab
     (1, 4608, 3072, 8, "", True, False),        # less than a slab
+    (1, 4096, 3072, 512, "", True, True),       # the double block's img tails: 256 tiles of 256 x 192, gated residual
+    (2, 2048, 3072, 200, "", False, True),      # K tail, two batch elements of eight tile rows each, no bias
+    (1, 2048, 6144, 136, "GELU", True, False),  # GELU on every column, 256 x 192
+    (1, 4096, 9216, 64, "", True, False),       # the double block's img qkv shape: three exact rounds, a single slab
+    (1, 4096, 3072, 8, "", True, False),        # less than a slab
 ])
 def test_linear_rectangular_tiles(B, L, N, K, act, bias, gated):
-    """Shapes that both 288 and 192 divide and that fill the 256 CUs better on 288 x 192 tiles than on
+    """Shapes that 288 x 192 or 256 x 192 tiles divide and that fill the 256 CUs better on them than on
     square ones take the rectangular-tile kernel: every epilogue it has, with and without a K tail."""
     g = seeded(B * L + N + K)
     M = B * L
@@ -103,6 +108,20 @@ def test_linear_rectangular_tiles(B, L, N, K, act, bias, gated):
     # and exactly the two PyTorch ops on the kernel's own (once rounded) product
     y = tk.linear(a, w, b)
     assert torch.equal(out, oracle.gated_residual_ref(x, gate, y.view(B, L, N)))
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 3072, 192), (4608, 3072, 200), (512, 3072, 256)])
+def test_linear_shared_gpu_flag_changes_the_schedule_only(M, N, K):
+    """FLUX_LINEAR_SHARED_GPU keeps the square tiles where the library would otherwise fill the CUs
+    exactly with rectangular ones; both orders of accumulation are the same, so are the bits."""
+    g = seeded(M + K)
+    a = randn(g, M, K, dtype=torch.bfloat16).to(DEV)
+    w = randn(g, N, K, dtype=torch.bfloat16, std=K ** -0.5).to(DEV)
+    b = randn(g, N, dtype=torch.bfloat16, std=0.5).to(DEV)
+    y0 = tk.linear_into(a, w, b, activation="GELU")
+    y1 = tk.linear_into(a, w, b, activation="GELU", shared_gpu=True)
+    assert torch.equal(y0, y1)
+    assert ((y1.float() - oracle.linear_ref_fp32(a, w, b, "GELU")).abs() <= half_ulp_bound(oracle.linear_ref_fp32(a, w, b, "GELU"))).all()
 
 
 def test_linear_unaligned_k_and_strided_input():

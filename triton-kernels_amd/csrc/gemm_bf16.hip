@@ -20,6 +20,7 @@
 // more and leaves as full 16-byte row segments, where the optional gated residual is applied.
 #include "common.h"
 #include <stdlib.h>
+#include <algorithm>
 #include <type_traits>
 
 namespace flux {
@@ -1217,16 +1218,16 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
-constexpr int kRectFM = 9, kRectFN = 6;   // 288 x 192 tiles
-
+// Rectangular tile shapes the host may pick: 288 x 192 and 256 x 192.
+template <int FM, int FN>
 static void launch_rect(GemmParams& p, hipStream_t st) {
-    constexpr int BM = 32 * kRectFM, BN = 32 * kRectFN;
+    constexpr int BM = 32 * FM, BN = 32 * FN;
     p.tiles_m = p.M / BM;
     p.tiles_n = p.N / BN;
     p.group_m = 4;
     const int grid = ((p.tiles_m * p.tiles_n + 7) / 8) * 8;
-    if (p.K % 64 == 0) hipLaunchKernelGGL((gemm_nt_rect_kernel<kRectFM, kRectFN, false>), dim3(grid), dim3(kGemmThreads), 0, st, p);
-    else hipLaunchKernelGGL((gemm_nt_rect_kernel<kRectFM, kRectFN, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    if (p.K % 64 == 0) hipLaunchKernelGGL((gemm_nt_rect_kernel<FM, FN, false>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    else hipLaunchKernelGGL((gemm_nt_rect_kernel<FM, FN, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
 }  // namespace flux
@@ -1241,6 +1242,7 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     if (a->M == 0 || a->N == 0) return FLUX_OK;
     if (a->lda < a->K || a->ldw < a->K) return fail(FLUX_E_SHAPE, "flux_linear_bf16: leading dimension smaller than K");
     if (a->act != FLUX_ACT_NONE && a->act != FLUX_ACT_GELU_TANH) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: unknown activation %d", a->act);
+    if ((a->flags & ~static_cast<int64_t>(FLUX_LINEAR_SHARED_GPU)) != 0) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: unknown flags 0x%llx", (unsigned long long)a->flags);
     if (a->in_act != FLUX_ACT_NONE && a->in_act != FLUX_ACT_SILU) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: unknown input activation %d", a->in_act);
     if (a->in_act == FLUX_ACT_SILU && (a->M > 8 || a->qk != nullptr)) return fail(FLUX_E_UNSUPPORTED, "flux_linear_bf16: input SiLU is for M <= 8 without the qk fusion (M=%lld)", (long long)a->M);
     const bool split = a->Y2 != nullptr && a->split_n < a->N;
@@ -1343,28 +1345,33 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
                 if ((fill == 0 || fill >= kGemmCUs * 9 / 10) && (p.gate == nullptr || (c * 256) % p.rows_per_batch == 0)) mb = c;
             }
         }
-        // 288 x 192 tiles when both extents divide and their rounds come out shorter than those of the
-        // square tiles. Measured at K = 3072: a round of square tiles 69 us, a round of 288 x 192 tiles
-        // 62 us (0.84 of the work at 1.06 times the cost per flop), a tail launch on 128-wide tiles
-        // 0.65 of a square round per wave of 512 workgroups plus a kernel boundary. 4608 x 3072 is
-        // 216 square tiles = one round with 40 CUs idle, and 256 tiles of 288 x 192; 4608 x 12288 is
-        // 3 square rounds and a tail, or 4 rounds of 288 x 192.
-        constexpr int RBM = 32 * kRectFM, RBN = 32 * kRectFN;
-        const bool rect_ok = p.M % RBM == 0 && p.N % RBN == 0 && p.vec_io && p.Y2 == nullptr &&
-                             (p.bias == nullptr || p.bias_vec) && (p.act == FLUX_ACT_NONE || p.act_begin == 0) &&
-                             (p.gate == nullptr || p.rows_per_batch % RBM == 0) &&
-                             a->lda * 2 * RBM < 0x7fffffffLL && a->ldw * 2 * RBN < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
-        if (rect_ok) {
+        // Rectangular tiles (288 x 192 or 256 x 192) when both extents divide and their rounds come out
+        // shorter than those of the square tiles. Measured at K = 3072: a round of square tiles 69 us,
+        // a round of 288 x 192 tiles 62 us (0.84 of the work at 1.06 times the cost per flop), a tail
+        // launch on 128-wide tiles 0.65 of a square round per wave of 512 workgroups plus a kernel
+        // boundary. 4608 x 3072 is 216 square tiles = one round with 40 CUs idle, and 256 tiles of
+        // 288 x 192; 4608 x 12288 is 3 square rounds and a tail, or 4 rounds of 288 x 192; 4096 x 3072
+        // is 192 square tiles, and 256 tiles of 256 x 192.
+        if (!(a->flags & FLUX_LINEAR_SHARED_GPU) && p.vec_io && p.Y2 == nullptr && (p.bias == nullptr || p.bias_vec) &&
+            (p.act == FLUX_ACT_NONE || p.act_begin == 0)) {
             double sq = static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
             if (mb) {
                 const int64_t rest_tiles = ((p.M - static_cast<int64_t>(mb) * 256 + 127) / 128) * ((p.N + 127) / 128);
                 sq = static_cast<double>((static_cast<int64_t>(mb) * tn + kGemmCUs - 1) / kGemmCUs) +
                      0.65 * static_cast<double>((rest_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)) + 0.1;
             }
-            const int64_t rt = static_cast<int64_t>(p.M / RBM) * (p.N / RBN);
-            const double rc = static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (RBM * RBN / 65536.0) * 1.06;
-            if (rc < 0.97 * sq) {
-                launch_rect(p, st);
+            // cost in square rounds of tiles of rbm x rbn, or a large number where they do not fit
+            auto rect_cost = [&](int rbm, int rbn) -> double {
+                const bool ok = p.M % rbm == 0 && p.N % rbn == 0 && (p.gate == nullptr || p.rows_per_batch % rbm == 0) &&
+                                a->lda * 2 * rbm < 0x7fffffffLL && a->ldw * 2 * rbn < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
+                if (!ok) return 1e30;
+                const int64_t rt = static_cast<int64_t>(p.M / rbm) * (p.N / rbn);
+                return static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (rbm * rbn / 65536.0) * 1.06;
+            };
+            const double c96 = rect_cost(288, 192), c86 = rect_cost(256, 192);
+            if (std::min(c96, c86) < 0.97 * sq) {
+                if (c96 <= c86) launch_rect<9, 6>(p, st);
+                else launch_rect<8, 6>(p, st);
                 return check_launch("flux_linear_bf16");
             }
         }

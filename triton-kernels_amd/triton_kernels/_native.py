@@ -17,6 +17,7 @@ _lib = None
 
 FLUX_BF16, FLUX_F32 = 0, 1
 ACT_NONE, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
+LINEAR_SHARED_GPU = 1
 E_NULL, E_SHAPE, E_DTYPE, E_ALIGN, E_TOO_WIDE, E_UNSUPPORTED = -1, -2, -3, -4, -5, -6
 MAX_ROW = 65536
 
@@ -61,6 +62,7 @@ class LinearArgs(Structure):
         ("ldresid", c_int64), ("gate_batch_stride", c_int64), ("rows_per_batch", c_int64),
         ("act", c_int32), ("in_act", c_int32), ("act_begin", c_int64),
         ("qk", POINTER(LinearQKFusion)),
+        ("flags", c_int64),
     ]
 
 
@@ -116,7 +118,7 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.flux_abi_version() != 3:
+        if handle.flux_abi_version() != 4:
             raise RuntimeError("libfluxhip.so: ABI version mismatch")
         _lib = handle
     return _lib
@@ -204,5 +206,5 @@ def src4(t: torch.Tensor | None) -> Src4:
 __all__ = [
     "lib", "lib_path", "check", "last_error", "dtype_code", "require_gpu", "stream_ptr", "on_device", "ptr", "src4",
     "Src4", "QkvPrepArgs", "LinearArgs", "AttnArgs", "SIGNATURES", "byref",
-    "FLUX_BF16", "FLUX_F32", "ACT_NONE", "ACT_GELU_TANH", "ACT_SILU", "MAX_ROW",
+    "FLUX_BF16", "FLUX_F32", "ACT_NONE", "ACT_GELU_TANH", "ACT_SILU", "LINEAR_SHARED_GPU", "MAX_ROW",
 ]

@@ -39,7 +39,7 @@ def _rows_2d(x: Tensor, K: int) -> Tensor:
 def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "", act_begin: int = 0,
                 out: Tensor | None = None, out2: Tensor | None = None, split: int | None = None,
                 resid: Tensor | None = None, gate: Tensor | None = None, qk: dict | None = None,
-                in_activation: str = "") -> Tensor:
+                in_activation: str = "", shared_gpu: bool = False) -> Tensor:
     """General form of the fused linear.
 
     out   : [M, >=split] destination (row stride free) for columns [0, split)
@@ -51,6 +51,9 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
             heads), which then go to q_out / k_out [B, heads, out_len, 128] instead of `out`:
             dict(q_out, k_out, q_scale, k_scale, pe, heads, seq_len, pos0=0, eps=1e-6); see
             qk_fusable() for the shapes this form takes
+    shared_gpu : the launch runs beside another stream's work; the library then keeps a tile shape
+            that leaves CUs free in its last round instead of one that fills the GPU exactly (same
+            result, only the schedule differs)
     """
     assert x.shape[-1] == w.shape[-1], "Incompatible dimensions"
     assert x.dtype == w.dtype, "Incompatible dtypes"
@@ -95,6 +98,7 @@ def linear_into(x: Tensor, w: Tensor, b: Tensor | None, *, activation: str = "",
         a.resid, a.ldresid = r2.data_ptr(), r2.stride(0)
         a.gate, a.gate_batch_stride, a.rows_per_batch = g2.data_ptr(), (g2.stride(0) if nb > 1 else N), M // nb
     a.act, a.act_begin = act, act_begin
+    a.flags = nv.LINEAR_SHARED_GPU if shared_gpu else 0
     a.in_act = {"": nv.ACT_NONE, "SiLU": nv.ACT_SILU}[in_activation]
     assert a.in_act == nv.ACT_NONE or M <= 8, "the input activation is fused for at most 8 rows"
     keep = None
@@ -136,7 +140,7 @@ def qk_fusable(x: Tensor, w: Tensor, seq_len: int, head_dim: int) -> bool:
             and N % 256 == 0 and w.shape[1] % 8 == 0 and -(-M // 256) * (N // 256) >= 160)
 
 
-def linear(x: Tensor, w: Tensor, b: Tensor | None, activation: str = "") -> Tensor:
+def linear(x: Tensor, w: Tensor, b: Tensor | None, activation: str = "", shared_gpu: bool = False) -> Tensor:
     N = w.shape[0]
-    y = linear_into(x, w, b, activation=activation)
+    y = linear_into(x, w, b, activation=activation, shared_gpu=shared_gpu)
     return y.reshape(*x.shape[:-1], N)

@@ -344,7 +344,7 @@ class DoubleStreamBlock(nn.Module):
         side.wait_stream(main)            # attention output is complete
         with torch.cuda.stream(side):
             self._stream_tail(txt, txt_attn, txt_mod1, txt_mod2, self.txt_attn.proj, self.txt_mlp, True, out=txt_out)
-        img = self._stream_tail(img, img_attn, img_mod1, img_mod2, self.img_attn.proj, self.img_mlp, True)
+        img = self._stream_tail(img, img_attn, img_mod1, img_mod2, self.img_attn.proj, self.img_mlp, True, beside_txt=True)
         main.wait_stream(side)
         # tensors made on the side stream that the caller's stream may still be reading when they die
         for t in (txt_mod1.shift, txt_mod1.scale, txt_mod1.gate, txt_mod2.shift, txt_mod2.scale, txt_mod2.gate):
@@ -353,7 +353,7 @@ class DoubleStreamBlock(nn.Module):
 
     @staticmethod
     def _stream_tail(x: Tensor, attn: Tensor, mod1: ModulationOut, mod2: ModulationOut, proj: Linear, mlp: nn.Sequential,
-                     fused: bool, out: Tensor | None = None) -> Tensor:
+                     fused: bool, out: Tensor | None = None, beside_txt: bool = False) -> Tensor:
         if not fused:
             x = _gated_residual(x, mod1.gate, proj(attn))
             return _gated_residual(x, mod2.gate, mlp(layer_norm_modulation(x, mod2.scale, mod2.shift)))
@@ -364,7 +364,11 @@ class DoubleStreamBlock(nn.Module):
         # attn is a slice of the [B, Lt+Li, hid] buffer: rows of one batch element are evenly strided,
         # batches are not, so flatten per call only when there is a single batch element.
         a2 = attn.reshape(M, hid) if B > 1 else attn[0]
-        linear_into(a2, proj.weight, proj.bias, out=x1.view(M, hid), resid=x.view(M, hid), gate=mod1.gate)
+        # beside_txt: the txt chain's projection runs on the other stream at the same time and lives on the
+        # CUs this launch leaves free (192 tiles at 4096 rows); a tile shape that fills all 256 CUs would
+        # push it behind. By the time of the last projection the txt chain has finished: measured at
+        # 4096 + 512 tokens, 1.18 ms like this, 1.23 ms with the flag on every launch or on none.
+        linear_into(a2, proj.weight, proj.bias, out=x1.view(M, hid), resid=x.view(M, hid), gate=mod1.gate, shared_gpu=beside_txt)
         h = linear(layer_norm_modulation(x1, mod2.scale, mod2.shift), mlp[0].weight, mlp[0].bias, activation="GELU")
         x2 = torch.empty_like(x) if out is None else out
         linear_into(h, mlp[2].weight, mlp[2].bias, out=x2.view(M, hid), resid=x1.view(M, hid), gate=mod2.gate)
