@@ -78,6 +78,34 @@ __device__ __forceinline__ u32x2 pack4_bf16(float a, float b, float c, float d) 
 // XCD w % 8; giving each XCD one contiguous range of the (grouped) tile sequence makes the ~32 tiles
 // resident on an XCD at any time a compact group_m x (32/group_m) patch that shares A and W panels
 // in that XCD's L2.
+// Tile order of a launch with the q/k epilogue. Its q/k tiles cost more than the others, each XCD
+// owns one contiguous range of the tile sequence and works through it alone, and in the natural
+// order one XCD would get twice its share of q/k tiles and another none. Here the q/k columns and
+// the other columns form two sequences (each grouped like the plain order, so that the tiles
+// resident on an XCD still share panels, and the q/k tiles of a patch the same rows of the rotation
+// table), and every XCD takes its eighth of the first followed by its eighth of the second.
+__device__ __forceinline__ bool tile_of_block_qk(const GemmParams& p, int bn, int& tm, int& tn) {
+    const int nq = p.qk_cols / bn;
+    const int Q = p.tiles_m * nq, R = p.tiles_m * (p.tiles_n - nq);
+    const int per_xcd = gridDim.x / 8;
+    const int x = blockIdx.x % 8, i = blockIdx.x / 8;
+    const int q0 = x * Q / 8, q1 = (x + 1) * Q / 8;
+    int u, cols, col0;
+    if (i < q1 - q0) {
+        u = q0 + i; cols = nq; col0 = 0;
+    } else {
+        u = x * per_xcd - q0 + (i - (q1 - q0)); cols = p.tiles_n - nq; col0 = nq;
+        if (u >= R) return false;
+    }
+    const int width = p.group_m * cols;
+    const int first_m = (u / width) * p.group_m;
+    const int gsz = min(p.tiles_m - first_m, p.group_m);
+    const int in_group = u % width;
+    tm = first_m + in_group % gsz;
+    tn = col0 + in_group / gsz;
+    return true;
+}
+
 __device__ __forceinline__ bool tile_of_block(const GemmParams& p, int& tm, int& tn) {
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = gridDim.x / 8;
@@ -750,7 +778,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
     constexpr int BM = 64 * MI, BK = 64, NU = 5, UNIT = BM * BK * 2;
     __shared__ __attribute__((aligned(1024))) char lds[NU * UNIT];
     int tm, tn;
-    if (!tile_of_block(p, tm, tn)) return;
+    if (p.qk_cols > 0 ? !tile_of_block_qk(p, BM, tm, tn) : !tile_of_block(p, tm, tn)) return;
     const int m0 = tm * BM, n0 = tn * BM;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
