@@ -194,7 +194,7 @@ int flux_linear_bf16(const flux_linear_args* args, void* stream);
  * relative error of at most 2^-8, so row i's base-2 scores, and with them lse, move by at most
  * 2^-8 * sm_scale * log2(e) * max_j sum_d |q_id k_jd|: a few 1e-3 for unit-variance inputs (o within
  * 4e-3 of the fp32 result at L = 4608), growing in proportion to |q| |k| (q thirty times larger:
- * lse up to 0.37 away, nearly one-hot outputs up to 0.25 at |v| ~ 4, 1e-2 on average). D = 16, 32
+ * lse up to 0.37 away, nearly one-hot outputs up to 0.33 at |v| ~ 4, 4e-3 on average). D = 16, 32
  * and 256 run a plain, unpipelined kernel that scales the fp32 scores.
  * ------------------------------------------------------------------------------------------- */
 typedef struct flux_attn_args {

@@ -120,7 +120,7 @@ def _prescaled_ref(q, k, v, sm_scale):
     return torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, dim=-1), v.float()), torch.logsumexp(s, -1) * math.log2(math.e)
 
 
-# (batch, heads, seq): which launch shape the head-dim-128 dispatch picks for them
+# (batch, heads, seq): which launch shape the head-dim-64/128 dispatch picks for them
 _WIDE = [(4, 24, 512),    # 64-row-per-wave kernel, one launch of 256-row tiles
          (4, 24, 1000),   # the same with a ragged last tile
          (1, 24, 4336),   # two launches (256- and 192-row tiles), ragged
@@ -135,10 +135,11 @@ _WIDE = [(4, 24, 512),    # 64-row-per-wave kernel, one launch of 256-row tiles
          (1, 25, 2300)]   # an odd head count with both tile sizes
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,H,L", _WIDE)
-def test_attention_wide_tile_launch_shapes(B, H, L):
-    g = seeded(B * 1000 + H * 100 + L)
-    q, k, v = (randn(g, B, H, L, 128, dtype=torch.bfloat16).to(DEV) for _ in range(3))
+def test_attention_wide_tile_launch_shapes(B, H, L, D):
+    g = seeded(B * 1000 + H * 100 + L + D)
+    q, k, v = (randn(g, B, H, L, D, dtype=torch.bfloat16).to(DEV) for _ in range(3))
     o = torch.empty_like(q)
     lse = torch.empty(B, H, L, dtype=torch.float32, device=DEV)
     tk.attention_into(q, k, v, o, lse=lse)
@@ -148,20 +149,22 @@ def test_attention_wide_tile_launch_shapes(B, H, L):
         torch.testing.assert_close(lse[b:b + 1], oracle.attention_lse_ref(q[b:b + 1], k[b:b + 1]), atol=5e-3, rtol=5e-4)
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("H", [24, 4])   # 24 heads: 64-row-per-wave kernel; 4 heads: 128-row workgroups
 @pytest.mark.parametrize("kind", ["hot", "ramp"])
-def test_attention_large_scores_move_the_reference_maximum(H, kind):
+def test_attention_large_scores_move_the_reference_maximum(H, kind, D):
     """Scores far above the first tile's maximum: the kernels subtract a per-row reference value that is
     only raised when a partial sum grows too large, and this drives them through that step."""
-    g = seeded(H + len(kind))
+    g = seeded(H + len(kind) + D)
     L = 2048
-    q = (randn(g, 1, H, L, 128) * (30.0 if kind == "hot" else 4.0)).bfloat16().to(DEV)
-    k = randn(g, 1, H, L, 128, dtype=torch.bfloat16).to(DEV)
-    v = randn(g, 1, H, L, 128, dtype=torch.bfloat16).to(DEV)
+    # the same spread of scores at either head dim: |q| grows as the head shrinks
+    q = (randn(g, 1, H, L, D) * ((30.0 if kind == "hot" else 4.0) * math.sqrt(128 / D))).bfloat16().to(DEV)
+    k = randn(g, 1, H, L, D, dtype=torch.bfloat16).to(DEV)
+    v = randn(g, 1, H, L, D, dtype=torch.bfloat16).to(DEV)
     if kind == "ramp":   # later keys score ever higher than earlier ones
         ramp = torch.linspace(0, 6.0, L, device=DEV).view(1, 1, L, 1)
         k = (k.float() + ramp * q.float().mean(dim=2, keepdim=True).sign()).bfloat16()
-    sc = 1 / math.sqrt(128)
+    sc = 1 / math.sqrt(128)   # at head dim 64 too: with the larger q the scores have the spread of the 128 case
     o = torch.empty_like(q)
     lse = torch.empty(1, H, L, dtype=torch.float32, device=DEV)
     tk.attention_into(q, k, v, o, sm_scale=sc, lse=lse)
@@ -176,13 +179,14 @@ def test_attention_large_scores_move_the_reference_maximum(H, kind):
     #     bound_i = 2^-8 * sm_scale * log2(e) * max_j sum_d |q_id| |k_jd|
     # which is a function of the input magnitudes only. The outputs of these nearly one-hot rows are
     # single v values (|v| up to ~4); their departure is bounded by what was measured when the kernel
-    # was written, with a third on top: 0.25 (hot) and 0.064 (ramp) at the maximum, ~1e-2 on average.
+    # was written, with a third on top: 0.24-0.33 (hot) and 0.047-0.066 (ramp) at the maximum over the
+    # four cases of either kind, 3.4e-3 and 1.8e-3 on average.
     lse_oracle = oracle.attention_lse_ref(q, k, sc)
     mag = torch.einsum("bhqd,bhkd->bhqk", q.float().abs(), k.float().abs()).amax(dim=-1)
     bound = mag * (sc * math.log2(math.e) * 2.0 ** -8)
     assert ((lse - lse_oracle).abs() <= bound + 1e-3).all()
     err = (o.float() - oracle.attention_ref_fp32(q, k, v, sc)).abs()
-    assert err.max().item() <= (0.33 if kind == "hot" else 0.085), err.max().item()
+    assert err.max().item() <= (0.44 if kind == "hot" else 0.088), err.max().item()
     assert err.mean().item() <= (2e-2 if kind == "hot" else 6e-3), err.mean().item()
 
 

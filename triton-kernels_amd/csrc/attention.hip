@@ -596,15 +596,20 @@ struct AttnSched {
 // QB = 16-row query blocks per wave: 16*QB slots, 4*QB units. With one wave per SIMD (QB = 4) a slot
 // takes one exponential or two other steps; with two waves per SIMD (QB = 2) the other wave fills
 // the gaps, there are fewer slots per step, and three other steps share a slot.
-template <int QB>
+// Head dim 64 has half the MFMAs per score: 8*QB slots for the same 8*QB exponentials, so every slot
+// carries one (the first four carry two, which lets the last units finish inside the iteration) and
+// up to two other steps behind it.
+template <int QB, int D>
 constexpr AttnSched attn_sched() {
-    constexpr int NS = 16 * QB, NE = 8 * QB, PER = QB >= 3 ? 2 : 3;
+    constexpr int NS = (D / 8) * QB, NE = 8 * QB, PER = QB >= 3 ? 2 : 3;
     AttnSched S{};
     int qk[160] = {}, qa[160] = {}, qr[160] = {};  // pending steps: kind, argument, first slot allowed
     int head = 0, tail = 0, next_exp = 0;
     for (int s = 0; s < NS; ++s) {
-        const bool exp_slot = s < 4 || s % 2 == 1;
-        if (exp_slot && next_exp < NE) {
+        const bool exp_slot = D == 64 || s < 4 || s % 2 == 1;
+        const int exps = !exp_slot ? 0 : (D == 64 && s < 4) ? 2 : 1;
+        int added = 0;
+        for (int e = 0; e < exps && next_exp < NE; ++e, ++added) {
             const int unit = next_exp / 2, second = next_exp % 2;
             S.kind[s][S.n[s]] = second ? ATT_E1 : ATT_E0; S.arg[s][S.n[s]] = unit; ++S.n[s];
             if (second) {
@@ -613,7 +618,8 @@ constexpr AttnSched attn_sched() {
                 if (unit % 4 != 0) { qk[tail] = ATT_A1; qa[tail] = unit; qr[tail] = s + 2; ++tail; }
             }
             ++next_exp;
-        } else {
+        }
+        if (D == 64 || added == 0) {
             for (int c = 0; c < PER && head < tail && qr[head] <= s; ++c) {
                 S.kind[s][S.n[s]] = qk[head]; S.arg[s][S.n[s]] = qa[head]; ++S.n[s]; ++head;
             }
@@ -627,17 +633,28 @@ constexpr AttnSched attn_sched() {
     S.kind[last][S.n[last]] = ATT_CHECK; S.arg[last][S.n[last]] = 0; ++S.n[last];
     return S;
 }
-template <int QB>
+template <int QB, int D>
 constexpr bool attn_sched_ok(int la) {  // every step exactly once, addresses ready before their first use
-    constexpr int NS = 16 * QB;
-    const AttnSched S = attn_sched<QB>();
+    constexpr int NS = (D / 8) * QB;
+    const AttnSched S = attn_sched<QB, D>();
     int seen[8][16] = {};
+    int exp_at[2][16] = {}, last_use[16] = {};   // position (slot * 8 + place in the slot) of a unit's exponentials and of its last other step
     for (int s = 0; s < NS; ++s) {
         if (S.n[s] > 8) return false;
         for (int c = 0; c < S.n[s]; ++c) {
-            seen[S.kind[s][c]][S.arg[s][c]] += 1;
+            const int kind = S.kind[s][c], u = S.arg[s][c];
+            seen[kind][u] += 1;
+            if (kind == ATT_E0 || kind == ATT_E1) exp_at[kind == ATT_E1][u] = s * 8 + c;
+            else if (kind != ATT_CHECK) {
+                last_use[u] = s * 8 + c;
+                // a step never shares a slot with the exponentials it reads
+                if (exp_at[0][u] / 8 == s || exp_at[1][u] / 8 == s) return false;
+            }
         }
     }
+    // the exponentials of four units are in flight at most: unit u + 4 reuses the registers of unit u
+    for (int u = 0; u + 4 < 4 * QB; ++u)
+        if (exp_at[0][u + 4] < last_use[u]) return false;
     for (int u = 0; u < 4 * QB; ++u) {
         if (seen[ATT_E0][u] != 1 || seen[ATT_E1][u] != 1 || seen[ATT_C][u] != 1 || seen[ATT_A0][u] != 1) return false;
         if (seen[ATT_A1][u] != (u % 4 != 0)) return false;
@@ -659,21 +676,28 @@ constexpr int attn_load_slot(int j, int ns, int bs, int sp, bool second) {
 //   <4, 4>: 64 rows per wave, 256 per workgroup, one wave per SIMD (248 vector + 192 accumulation registers).
 //   <3, 4>: 48 rows per wave, 192 per workgroup: the same code with three quarters of the work per
 //           iteration, for the part that evens out the last round (see attn_launch_w64).
-template <int QB, int NW>
+//
+// Head dim 64 runs the same code with half the MFMAs per iteration (2 + 2 fragments of K, 4 of V^T per
+// 32 keys) and the same softmax work, so there the VALU sets the pace: every slot carries an
+// exponential. Rows of K and V are 128 bytes, a wave-wide load covers eight of them, and the swizzles
+// are those of 128-byte rows (below).
+template <int D, int QB, int NW>
 __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, const int block, const int nblocks) {
-    static_assert(NW == 4 && (QB == 3 || QB == 4), "configurations that have been laid out and measured");
+    static_assert(NW == 4 && (QB == 3 || QB == 4) && (D == 64 || D == 128), "configurations that have been laid out and measured");
     constexpr int ROWS = 16 * QB * NW;         // query rows per workgroup
-    constexpr int D = 128, KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
+    constexpr int KS = D / 32, DBN = D / 16, ROWB = D * 2, TB = 64 * ROWB, HALF = 32 * ROWB;
+    constexpr int CH = D / 8, RPL = 64 / CH;   // 16-byte chunks per row; rows a wave-wide load (or store) covers
     constexpr int V0 = 4 * TB;
-    constexpr int NS = 16 * QB, NSS = 8 * QB;  // MFMA slots per iteration; the first NSS are S^T
+    constexpr int NSS = 2 * KS * QB, NS = NSS + DBN * QB;  // MFMA slots per iteration; the first NSS are S^T
     constexpr int LA = 3 * QB;                 // look-ahead of the LDS fragment reads in slots: what a ring of four fragments holds
-    constexpr int BS = 10 * QB;                // slot of the barrier in the first iteration of a body
-    constexpr int PP = 16 / NW;                // loader passes per tile and operand (a pass = 4 rows per wave)
+    constexpr int BS = D == 128 ? 10 * QB : 4 * QB;  // slot of the barrier in the first iteration of a body
+    constexpr int PP = 64 / (RPL * NW);        // loader passes per tile and operand (a pass = RPL rows per wave)
     constexpr int LPW = 2 * PP;                // buffer loads per wave and body: PP of V(T+2), then PP of K(T+4)
-    constexpr int kAccQ = 32 * QB;             // first accumulation register of the Q fragments
-    constexpr AttnSched SCHED = attn_sched<QB>();
-    static_assert(attn_sched_ok<QB>(LA), "VALU schedule");
-    static_assert(BS > 7 * QB - LA && BS < NS - LA, "barrier between the last read of K(T) and the first of K(T+1)");
+    constexpr int kAccQ = 4 * DBN * QB;        // first accumulation register of the Q fragments
+    constexpr int kQRegs = 4 * KS;             // accumulation registers of one query block's fragments
+    constexpr AttnSched SCHED = attn_sched<QB, D>();
+    static_assert(attn_sched_ok<QB, D>(LA), "VALU schedule");
+    static_assert(BS > (2 * KS - 1) * QB - LA && BS < NS - LA, "barrier between the last read of K(T) and the first of K(T+1)");
     static_assert(attn_load_slot(LPW - 1, NS, BS, NS / 8, false) != -2, "load slots");
     constexpr float kRebase = 1.0995116e12f;  // 2^40
     // lds: 8 * TB bytes, K ring of 4 tiles, V ring of 4 tiles
@@ -695,17 +719,21 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     const bf16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
     const bf16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
 
-    // loader: a wave-wide load is 4 rows x 256 bytes; pass i covers rows i*4*NW + wave*4 + lane/16.
-    // LDS position pos of row r holds the 16-byte chunk pos ^ (r & 15) of a K row (fragment reads
-    // take one chunk of 16 consecutive rows) and chunk pos ^ ((r & 7) << 1) of a V row (transposing
-    // reads take 32-byte pieces of 4 consecutive rows in each of four lane groups).
-    const int l_row = lane >> 4, l_pos = lane & 15;
+    // loader: a wave-wide load is RPL rows of ROWB bytes (1 KB); pass i covers rows i*RPL*NW + wave*RPL + lane/CH.
+    // 256-byte rows: LDS position pos of row r holds the 16-byte chunk pos ^ (r & 15) of a K row
+    // (fragment reads take one chunk of 16 consecutive rows) and chunk pos ^ ((r & 7) << 1) of a V row
+    // (transposing reads take 32-byte pieces of 4 consecutive rows in each of four lane groups).
+    // 128-byte rows: two rows fill the 256 bytes the banks are wide, so the rows of a pair keep the
+    // same position and the pairs differ: chunk pos ^ ((r >> 1) & 7) for K, pos ^ (((r >> 1) & 3) << 1) for V.
+    auto k_swz = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto v_swz = [](int r) { return D == 128 ? (r & 7) : ((r >> 1) & 3); };   // in 32-byte units
+    const int l_row = lane / CH, l_pos = lane % CH;
     uint32_t k_voff[PP], v_voff[PP];
 #pragma unroll
     for (int i = 0; i < PP; ++i) {
-        const int r = i * 4 * NW + wave * 4 + l_row;
-        k_voff[i] = static_cast<uint32_t>((r * p.k_sl + ((l_pos ^ (r & 15)) * 8)) * 2);
-        v_voff[i] = static_cast<uint32_t>((r * p.v_sl + ((l_pos ^ ((r & 7) << 1)) * 8)) * 2);
+        const int r = i * RPL * NW + wave * RPL + l_row;
+        k_voff[i] = static_cast<uint32_t>((r * p.k_sl + ((l_pos ^ k_swz(r)) * 8)) * 2);
+        v_voff[i] = static_cast<uint32_t>((r * p.v_sl + ((l_pos ^ (v_swz(r) << 1)) * 8)) * 2);
     }
     const int k_row2 = static_cast<int>(p.k_sl * 2), v_row2 = static_cast<int>(p.v_sl * 2);
     auto tile_rsrc = [&](const bf16_t* base, int row2, int key0) -> u32x4 {
@@ -736,7 +764,7 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     {
         const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int i = 0; i < 16 / NW; ++i) *reinterpret_cast<u32x4*>(lds + V0 + 3 * TB + i * (NW * 1024) + tid * 16) = z;
+        for (int i = 0; i < PP; ++i) *reinterpret_cast<u32x4*>(lds + V0 + 3 * TB + i * (NW * 1024) + tid * 16) = z;
     }
     load_k(0, 0);
     load_v(0, 0);
@@ -744,9 +772,9 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
 
     // Q fragments ("B" operand of S^T): lane holds row q0 + qb*16 + r16, d = ks*32 + g*8 .. +8,
     // scaled by sm_scale*log2(e) and rounded to bf16.
-    attn_claim_agprs<48 * QB>();
+    attn_claim_agprs<(D == 128 ? 48 * QB : 96)>();
     {
-        u32x4 qraw[QB][KS];  // all sixteen loads in flight before the first conversion
+        u32x4 qraw[QB][KS];  // all loads in flight before the first conversion
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
             const int row = q0 + qb * 16 + r16;
@@ -759,11 +787,11 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
             }
         }
         static_for<0, QB * KS * 4>([&](auto i_c) {
-            constexpr int i = decltype(i_c)::value, qb = i / 16, ks = (i / 4) % 4, e = i % 4;
+            constexpr int i = decltype(i_c)::value, qb = i / kQRegs, ks = (i / 4) % KS, e = i % 4;
             const uint32_t t = qraw[qb][ks][e];
             acc_write<kAccQ + i>(pack2_bf16(__uint_as_float(t << 16) * c, __uint_as_float(t & 0xffff0000u) * c));
         });
-        static_for<0, 32 * QB>([&](auto i_c) { acc_write<decltype(i_c)::value>(0u); });  // O^T = 0
+        static_for<0, kAccQ>([&](auto i_c) { acc_write<decltype(i_c)::value>(0u); });  // O^T = 0
     }
 
     // fragment addresses, lane part (the ring offset of the sub-tile is added once per iteration,
@@ -773,11 +801,11 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     // (second read) of the sub-tile; lane r16 points at row g*4 + r16/4, 8 bytes at d = db*16 + (r16%4)*4.
     int k_addr[KS], v_addr[DBN];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = r16 * ROWB + (((ks * 4 + g) ^ r16) * 16);
+    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = r16 * ROWB + (((ks * 4 + g) ^ k_swz(r16)) * 16);
     {
         const int rr = r16 >> 2, cc = r16 & 3, row = g * 4 + rr;
 #pragma unroll
-        for (int db = 0; db < DBN; ++db) v_addr[db] = V0 + row * ROWB + ((db ^ (row & 7)) * 32) + cc * 8;
+        for (int db = 0; db < DBN; ++db) v_addr[db] = V0 + row * ROWB + ((db ^ v_swz(row)) * 32) + cc * 8;
     }
 
     f32x4 seed[QB];   // -m of the row, in every register of the block: C operand of the first S^T MFMA
@@ -808,9 +836,9 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
         for (int w = 0; w < 4; ++w) pw0[qb][w] = pw1[qb][w] = 0u;
         s0[0][qb] = s0[1][qb] = s1[0][qb] = s1[1][qb] = zero4;
     }
-    auto read_k = [&](int off, int n) {  // n-th K fragment of the sub-tile at LDS offset off (a constant): key block n/4, d step n%4
+    auto read_k = [&](int off, int n) {  // n-th K fragment of the sub-tile at LDS offset off (a constant): key block n/KS, d step n%KS
         keep_regs(kf[n % 4]);
-        kf[n % 4] = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % 4] + (off + (n / 4) * 16 * ROWB));
+        kf[n % 4] = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % KS] + (off + (n / KS) * 16 * ROWB));
     };
     auto vfrag = [&](int m) {
         typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -820,17 +848,15 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
 
     // ---- prologue: S^T(0) from the first half of K(0), then the rows' first reference maxima
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#pragma unroll
-    for (int n = 0; n < 8; ++n) {
-        const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + k_addr[n % 4] + (n / 4) * 16 * ROWB);
+    static_for<0, 2 * KS>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value, kb = n / KS, ks = n % KS;
+        const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + k_addr[ks] + kb * 16 * ROWB);
         static_for<0, QB>([&](auto qb_c) {
-            constexpr int qb = decltype(qb_c)::value, QA = 32 * QB + 16 * qb;
-            if (n % 4 == 0) mfma_s_zero<QA>(s0[n / 4][qb], f);
-            else if (n % 4 == 1) mfma_s_acc<QA + 4>(s0[n / 4][qb], f);
-            else if (n % 4 == 2) mfma_s_acc<QA + 8>(s0[n / 4][qb], f);
-            else mfma_s_acc<QA + 12>(s0[n / 4][qb], f);
+            constexpr int qb = decltype(qb_c)::value, QA = kAccQ + kQRegs * qb;
+            if constexpr (ks == 0) mfma_s_zero<QA>(s0[kb][qb], f);
+            else mfma_s_acc<QA + 4 * ks>(s0[kb][qb], f);
         });
-    }
+    });
     mfma_settle(s0);
     load_k(2, 2);
     load_v(1, 1);
@@ -929,9 +955,9 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
             }
             // ---- matrix pipe
             if constexpr (i < NSS) {
-                constexpr int n = i / QB, qb = i % QB, kb = n / 4, ks = n % 4;
-                if constexpr (ks == 0) mfma_s_seed<kAccQ + 16 * qb>(sn[kb][qb], kf[n % 4], seed[qb]);
-                else mfma_s_acc<kAccQ + 16 * qb + 4 * ks>(sn[kb][qb], kf[n % 4]);
+                constexpr int n = i / QB, qb = i % QB, kb = n / KS, ks = n % KS;
+                if constexpr (ks == 0) mfma_s_seed<kAccQ + kQRegs * qb>(sn[kb][qb], kf[n % 4], seed[qb]);
+                else mfma_s_acc<kAccQ + kQRegs * qb + 4 * ks>(sn[kb][qb], kf[n % 4]);
             } else {
                 constexpr int m = (i - NSS) / QB, qb = i % QB;
                 mfma_o_acc<4 * (m * QB + qb)>(vfrag(m % 4), ppf[qb]);
@@ -941,15 +967,15 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
             // an iteration are read in the one before)
             static_for<0, 8>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value;
-                if constexpr (QB * n - LA == i) read_k(KC, n);
-                if constexpr (NS + QB * n - LA == i) read_k(KN, n);
-                if constexpr (NSS + QB * n - LA == i) {
+                if constexpr (n < 2 * KS && QB * n - LA == i) read_k(KC, n);
+                if constexpr (n < 2 * KS && NS + QB * n - LA == i) read_k(KN, n);
+                if constexpr (n < DBN && NSS + QB * n - LA == i) {
                     keep_regs(vlo[n % 4]);
-                    vlo[n % 4] = lds_read_tr(lds + v_addr[n] + VC);
+                    vlo[n % 4] = lds_read_tr(lds + v_addr[n % DBN] + VC);
                 }
-                if constexpr (NSS + 1 + QB * n - LA == i) {
+                if constexpr (n < DBN && NSS + 1 + QB * n - LA == i) {
                     keep_regs(vhi[n % 4]);
-                    vhi[n % 4] = lds_read_tr(lds + v_addr[n] + (VC + 16 * ROWB));
+                    vhi[n % 4] = lds_read_tr(lds + v_addr[n % DBN] + (VC + 16 * ROWB));
                 }
             });
             // ---- global loads of later tiles behind the barrier
@@ -1066,7 +1092,7 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     // ---- finish: fold the four lane groups' partial sums, normalise, store. A lane holds runs of four
     // columns of sixteen different rows, which would leave as 32-byte pieces; instead the wave parks
     // its rows in LDS (the rings are idle once every wave is past the loop) and they leave as 16-byte
-    // pieces of whole 256-byte rows. 8-byte slot s of row r sits at slot s ^ 2(r & 15): writes and
+    // pieces of whole rows. 8-byte slot s of row r sits at slot s ^ 2(r mod chunks per row): writes and
     // reads both spread over all banks, and a 16-byte chunk stays contiguous.
     asm volatile("s_barrier" ::: "memory");
     char* const stage = lds + wave * (16 * QB * ROWB);
@@ -1082,7 +1108,7 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
             u32x2 w;
             w.x = pack2_bf16(acc_read<r>() * inv, acc_read<r + 1>() * inv);
             w.y = pack2_bf16(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
-            *reinterpret_cast<u32x2*>(srow + (((db * 4 + g) ^ (r16 * 2)) * 8)) = w;
+            *reinterpret_cast<u32x2*>(srow + (((db * 4 + g) ^ ((r16 % CH) * 2)) * 8)) = w;
         });
         if (row < p.L && p.lse != nullptr && g == 0)
             p.lse[static_cast<int64_t>(bh) * p.L + row] = -seed[qb][0] + __builtin_amdgcn_logf(l_tot);
@@ -1090,11 +1116,11 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
     __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
     {
         bf16_t* const obase = p.o + b * p.o_sb + h * p.o_sh;
-        const int chunk = lane & 15;
+        const int chunk = lane % CH;
 #pragma unroll
-        for (int it = 0; it < 4 * QB; ++it) {
-            const int rl = it * 4 + (lane >> 4);
-            const u32x4 y = *reinterpret_cast<const u32x4*>(stage + rl * ROWB + ((chunk ^ (rl & 15)) * 16));
+        for (int it = 0; it < 16 * QB / RPL; ++it) {
+            const int rl = it * RPL + lane / CH;
+            const u32x4 y = *reinterpret_cast<const u32x4*>(stage + rl * ROWB + ((chunk ^ (rl % CH)) * 16));
             const int row = q0 + rl;
             if (row < p.L) *reinterpret_cast<u32x4*>(obase + static_cast<int64_t>(row) * p.o_sl + chunk * 8) = y;
         }
@@ -1102,22 +1128,23 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
 }
 
 
-constexpr int kW64LdsBytes = 8 * 64 * 256;  // K ring and V ring of four 64-key tiles of 256-byte rows
+constexpr int w64_lds_bytes(int d) { return 8 * 64 * 2 * d; }  // K ring and V ring of four 64-key tiles
 
-template <int QB, int NW>
+template <int D, int QB, int NW>
 __global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(1024))) char lds[kW64LdsBytes];
-    attn_w64_tile<QB, NW>(p, lds, blockIdx.x, gridDim.x);
+    __shared__ __attribute__((aligned(1024))) char lds[w64_lds_bytes(D)];
+    attn_w64_tile<D, QB, NW>(p, lds, blockIdx.x, gridDim.x);
 }
 
 // Both tile sizes in one launch: blocks [0, n4) take 256-row tiles of p4, the rest 192-row tiles of
 // p3. Workgroups are handed out in order, so the 192-row tiles start on each CU as it finishes its
 // 256-row tile, with no launch boundary in between. n4 and the remainder are multiples of eight, so
 // a block's XCD is the same counted from either start.
+template <int D>
 __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel_pair(AttnParams p4, AttnParams p3, int n4) {
-    __shared__ __attribute__((aligned(1024))) char lds[kW64LdsBytes];
-    if (static_cast<int>(blockIdx.x) < n4) attn_w64_tile<4, 4>(p4, lds, blockIdx.x, n4);
-    else attn_w64_tile<3, 4>(p3, lds, static_cast<int>(blockIdx.x) - n4, static_cast<int>(gridDim.x) - n4);
+    __shared__ __attribute__((aligned(1024))) char lds[w64_lds_bytes(D)];
+    if (static_cast<int>(blockIdx.x) < n4) attn_w64_tile<D, 4, 4>(p4, lds, blockIdx.x, n4);
+    else attn_w64_tile<D, 3, 4>(p3, lds, static_cast<int>(blockIdx.x) - n4, static_cast<int>(gridDim.x) - n4);
 }
 
 template <int D, int QB, int BN>
@@ -1201,6 +1228,7 @@ static void attn_w64_cut(int64_t BH, int L, int& best_ne, int& best_no) {
     if (filled < 8) ++filled;
 }
 
+template <int D>
 static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
     const int n256 = (p.L + 255) / 256;
     const int64_t tiles = BH * n256;
@@ -1216,12 +1244,12 @@ static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
             AttnParams p4 = p, p3 = p;
             const int g4 = attn_w64_part(p4, BH, best_ne, best_no, 0, 0);
             const int g3 = attn_w64_part(p3, BH, (p.L - fe + 191) / 192, (p.L - fo + 191) / 192, fe, fo);
-            hipLaunchKernelGGL(attn_fwd_w64_kernel_pair, dim3(g4 + g3), dim3(256), 0, st, p4, p3, g4);
+            hipLaunchKernelGGL(attn_fwd_w64_kernel_pair<D>, dim3(g4 + g3), dim3(256), 0, st, p4, p3, g4);
             return;
         }
     }
     const int g = attn_w64_part(p, BH, n256, n256, 0, 0);
-    if (g > 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<4, 4>), dim3(g), dim3(256), 0, st, p);
+    if (g > 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<D, 4, 4>), dim3(g), dim3(256), 0, st, p);
 }
 
 }  // namespace flux
@@ -1262,8 +1290,9 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
     if (a->D != 64 && a->D != 128) {
         if (BH * ((a->L + 63) / 64) > 0x7fffffffLL) return fail(FLUX_E_SHAPE, "flux_attention_fwd_bf16: problem too large");
         attn_launch_plain(p, BH, a->D, st);
-    } else if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64(p, BH, st);
+    } else if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64<128>(p, BH, st);
     else if (a->D == 128) attn_launch_pipe<128, 1, 64>(p, BH, st);
+    else if (tiles256 >= kW64MinTiles) attn_launch_w64<64>(p, BH, st);
     else attn_launch_pipe<64, 1, 64>(p, BH, st);
     return check_launch("flux_attention_fwd_bf16");
 }
