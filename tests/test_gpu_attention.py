@@ -150,6 +150,22 @@ def test_attention_wide_tile_launch_shapes(B, H, L, D):
 
 
 @pytest.mark.parametrize("D", [128, 64])
+def test_attention_wide_tile_strided_views(D):
+    """The 64-row-per-wave kernels on views of a packed qkv projection (row stride 3 * H * D) with the
+    output written head-interleaved, as the blocks pass them, ragged length, with lse."""
+    g = seeded(7 + D)
+    B, H, L = 2, 3072 // D, 1100
+    qkv = randn(g, B, L, 3 * H * D, dtype=torch.bfloat16).to(DEV)
+    q, k, v = oracle.split_heads_ref(qkv, H)
+    out = torch.empty(B, L, H, D, dtype=torch.bfloat16, device=DEV).permute(0, 2, 1, 3)
+    lse = torch.empty(B, H, L, dtype=torch.float32, device=DEV)
+    tk.attention_into(q, k, v, out, lse=lse)
+    for b in range(B):
+        torch.testing.assert_close(out[b:b + 1].float(), oracle.attention_ref_fp32(q[b:b + 1], k[b:b + 1], v[b:b + 1]), atol=1e-2, rtol=0)
+        torch.testing.assert_close(lse[b:b + 1], oracle.attention_lse_ref(q[b:b + 1], k[b:b + 1]), atol=5e-3, rtol=5e-4)
+
+
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("H", [24, 4])   # 24 heads: 64-row-per-wave kernel; 4 heads: 128-row workgroups
 @pytest.mark.parametrize("kind", ["hot", "ramp"])
 def test_attention_large_scores_move_the_reference_maximum(H, kind, D):
