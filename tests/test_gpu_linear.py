@@ -83,6 +83,7 @@ def test_linear_ragged_shapes(M, N, K, bias):
     (1, 2048, 6144, 136, "GELU", True, False),  # GELU on every column, 256 x 192
     (1, 4096, 9216, 64, "", True, False),       # the double block's img qkv shape: three exact rounds, a single slab
     (1, 4096, 3072, 8, "", True, False),        # less than a slab
+    (1, 2816, 3072, 320, "GELU", True, False),  # too few square tiles, two rounds of 128-wide ones: 176 tiles of 256 x 192
 ])
 def test_linear_rectangular_tiles(B, L, N, K, act, bias, gated):
     """Shapes that 288 x 192 or 256 x 192 tiles divide and that fill the 256 CUs better on them than on

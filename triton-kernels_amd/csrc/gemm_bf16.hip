@@ -1356,6 +1356,32 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     // 256-wide tiles once they fill most of the chip; below that 128-wide ones (two workgroups per
     // CU); problems with too few of those to give every second CU one are bound by the latency of
     // the K loop and run on 64-wide tiles, four times as many workgroups.
+    // Rectangular tiles (288 x 192 or 256 x 192) when both extents divide and their rounds come out
+    // shorter than those of the other tiles. Measured at K = 3072: a round of square tiles 69 us, a
+    // round of 288 x 192 tiles 62 us (0.84 of the work at 1.06 times the cost per flop), a launch on
+    // 128-wide tiles 0.57 to 0.65 of a square round per wave of 512 workgroups, plus a kernel boundary
+    // when it is the tail of a split launch. 4608 x 3072 is 216 square tiles = one round with 40 CUs
+    // idle, and 256 tiles of 288 x 192; 4608 x 12288 is 3 square rounds and a tail, or 4 rounds of
+    // 288 x 192; 4096 x 3072 is 192 square tiles, and 256 tiles of 256 x 192; 2816 x 3072 is two
+    // rounds of 128-wide tiles, the second nearly empty, and 176 tiles of 256 x 192.
+    const bool rect_form = !(a->flags & FLUX_LINEAR_SHARED_GPU) && p.vec_io && p.Y2 == nullptr && (p.bias == nullptr || p.bias_vec) &&
+                           (p.act == FLUX_ACT_NONE || p.act_begin == 0);
+    // cost in square rounds of tiles of rbm x rbn, or a large number where they do not fit
+    auto rect_cost = [&](int rbm, int rbn) -> double {
+        const bool ok = rect_form && p.M % rbm == 0 && p.N % rbn == 0 && (p.gate == nullptr || p.rows_per_batch % rbm == 0) &&
+                        a->lda * 2 * rbm < 0x7fffffffLL && a->ldw * 2 * rbn < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
+        if (!ok) return 1e30;
+        const int64_t rt = static_cast<int64_t>(p.M / rbm) * (p.N / rbn);
+        return static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (rbm * rbn / 65536.0) * 1.06;
+    };
+    // launches on the cheaper rectangular shape if that costs less than `other` (in square rounds)
+    auto rect_if_cheaper = [&](double other) -> bool {
+        const double c96 = rect_cost(288, 192), c86 = rect_cost(256, 192);
+        if (!(std::min(c96, c86) < 0.97 * other)) return false;
+        if (c96 <= c86) launch_rect<9, 6>(p, st);
+        else launch_rect<8, 6>(p, st);
+        return true;
+    };
     if (big_tiles >= 160) {
         // One workgroup per CU: a launch whose last round is mostly empty pays for a whole round
         // (864 tiles of mlp_in at 4608 rows = 3.375 rounds cost 4). When a leading block of whole
@@ -1373,36 +1399,13 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
                 if ((fill == 0 || fill >= kGemmCUs * 9 / 10) && (p.gate == nullptr || (c * 256) % p.rows_per_batch == 0)) mb = c;
             }
         }
-        // Rectangular tiles (288 x 192 or 256 x 192) when both extents divide and their rounds come out
-        // shorter than those of the square tiles. Measured at K = 3072: a round of square tiles 69 us,
-        // a round of 288 x 192 tiles 62 us (0.84 of the work at 1.06 times the cost per flop), a tail
-        // launch on 128-wide tiles 0.65 of a square round per wave of 512 workgroups plus a kernel
-        // boundary. 4608 x 3072 is 216 square tiles = one round with 40 CUs idle, and 256 tiles of
-        // 288 x 192; 4608 x 12288 is 3 square rounds and a tail, or 4 rounds of 288 x 192; 4096 x 3072
-        // is 192 square tiles, and 256 tiles of 256 x 192.
-        if (!(a->flags & FLUX_LINEAR_SHARED_GPU) && p.vec_io && p.Y2 == nullptr && (p.bias == nullptr || p.bias_vec) &&
-            (p.act == FLUX_ACT_NONE || p.act_begin == 0)) {
-            double sq = static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
-            if (mb) {
-                const int64_t rest_tiles = ((p.M - static_cast<int64_t>(mb) * 256 + 127) / 128) * ((p.N + 127) / 128);
-                sq = static_cast<double>((static_cast<int64_t>(mb) * tn + kGemmCUs - 1) / kGemmCUs) +
-                     0.65 * static_cast<double>((rest_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)) + 0.1;
-            }
-            // cost in square rounds of tiles of rbm x rbn, or a large number where they do not fit
-            auto rect_cost = [&](int rbm, int rbn) -> double {
-                const bool ok = p.M % rbm == 0 && p.N % rbn == 0 && (p.gate == nullptr || p.rows_per_batch % rbm == 0) &&
-                                a->lda * 2 * rbm < 0x7fffffffLL && a->ldw * 2 * rbn < 0x7fffffffLL;   // 32-bit byte offsets inside a tile's rows
-                if (!ok) return 1e30;
-                const int64_t rt = static_cast<int64_t>(p.M / rbm) * (p.N / rbn);
-                return static_cast<double>((rt + kGemmCUs - 1) / kGemmCUs) * (rbm * rbn / 65536.0) * 1.06;
-            };
-            const double c96 = rect_cost(288, 192), c86 = rect_cost(256, 192);
-            if (std::min(c96, c86) < 0.97 * sq) {
-                if (c96 <= c86) launch_rect<9, 6>(p, st);
-                else launch_rect<8, 6>(p, st);
-                return check_launch("flux_linear_bf16");
-            }
+        double sq = static_cast<double>((big_tiles + kGemmCUs - 1) / kGemmCUs);
+        if (mb) {
+            const int64_t rest_tiles = ((p.M - static_cast<int64_t>(mb) * 256 + 127) / 128) * ((p.N + 127) / 128);
+            sq = static_cast<double>((static_cast<int64_t>(mb) * tn + kGemmCUs - 1) / kGemmCUs) +
+                 0.65 * static_cast<double>((rest_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)) + 0.1;
         }
+        if (rect_if_cheaper(sq)) return check_launch("flux_linear_bf16");
         if (mb == 0) {
             launch_tiled<4>(p, st);
         } else {
@@ -1420,6 +1423,6 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
         }
     }
     else if (mid_tiles <= 64) launch_tiled<1>(p, st);
-    else launch_tiled<2>(p, st);
+    else if (!rect_if_cheaper(0.57 * static_cast<double>((mid_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)))) launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
 }
