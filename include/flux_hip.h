@@ -176,8 +176,10 @@ typedef struct flux_linear_args {
 
 /* flags: the launch will run beside work of another stream (the txt chain beside the img chain of
  * the double-stream block). The library then keeps the tile shape whose last round leaves CUs free
- * for that work instead of the one that fills every round of the 256 CUs exactly, which is the
- * faster one only when the launch has the GPU to itself. The result is the same bits either way. */
+ * for that work instead of the one that fills every round of the 256 CUs exactly, and gives a
+ * small problem few, larger workgroups instead of one or two on every CU; both other choices are
+ * the faster ones only when the launch has the GPU to itself. The result is the same bits either
+ * way. */
 #define FLUX_LINEAR_SHARED_GPU 1
 
 int flux_linear_bf16(const flux_linear_args* args, void* stream);

@@ -788,6 +788,105 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_ring_kernel(GemmParams p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Few tiles: a launch that cannot fill the CUs with 256-wide tiles is bound by the latency of its K
+// loop, above all when the weights come from HBM (the first use in a forward pass): a workgroup then
+// waits for every slab in turn, and what counts is how many slabs it has in flight. The ring above
+// keeps one and a half; this kernel keeps ST - 1 whole slabs (A and W) of a 64*MI-wide tile in LDS
+// buffers used round-robin, with one barrier per slab: behind the barrier of slab kt the buffer of slab
+// kt - 1 takes slab kt + ST - 1. Fragment reads and MFMAs are left to the compiler's scheduler: the
+// loop waits on memory, not on issue slots.
+// ------------------------------------------------------------------------------------------------
+template <int MI, int ST, bool KTAIL>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_deep_kernel(GemmParams p) {
+    constexpr int FM = 2 * MI, FN = 2 * MI;
+    constexpr int BM = 64 * MI, BK = 64, ROWB = BK * 2, KSUB = BK / 32;
+    constexpr int UNIT = BM * ROWB, SLAB = 2 * UNIT;   // a slab: A rows, then W rows
+    constexpr int PU = BM / 32, NL = 2 * PU;           // buffer loads per thread per operand / per slab
+    constexpr int WROWS = 32 * MI;
+    static_assert(ST >= 3 && (ST - 2) * NL <= 63 && ST * SLAB <= 160 * 1024 && 4 * WROWS * WROWS * 2 <= ST * SLAB, "ring shape");
+    __shared__ __attribute__((aligned(1024))) char lds[ST * SLAB];
+    int tm, tn;
+    if (!tile_of_block(p, tm, tn)) return;
+    const int m0 = tm * BM, n0 = tn * BM;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // loader mapping and swizzle as in gemm_tile_slabs
+    const int lrow = tid >> 3;
+    const int lchunk = (tid & 7) ^ ((lrow >> 1) & 7);
+    const int rows_a = min(p.M - m0, BM), rows_b = min(p.N - n0, BM);
+    bf16_t* const base_a = const_cast<bf16_t*>(p.A + static_cast<int64_t>(m0) * p.lda);
+    bf16_t* const base_b = const_cast<bf16_t*>(p.W + static_cast<int64_t>(n0) * p.ldw);
+    const int bytes_a = static_cast<int>(((rows_a - 1) * p.lda + p.K) * 2);
+    const int bytes_b = static_cast<int>(((rows_b - 1) * p.ldw + p.K) * 2);
+    uint32_t voff_a[PU], voff_b[PU];
+#pragma unroll
+    for (int i = 0; i < PU; ++i) {
+        const int r = i * 32 + lrow;
+        voff_a[i] = r < rows_a ? static_cast<uint32_t>((r * p.lda + lchunk * 8) * 2) : kOutOfRange;
+        voff_b[i] = r < rows_b ? static_cast<uint32_t>((r * p.ldw + lchunk * 8) * 2) : kOutOfRange;
+    }
+    const int ke = (p.K + BK - 1) / BK;
+    // slabs past the end read as zeros (and keep the count of loads in flight the same to the last slab)
+    auto load_slab = [&](int soff, int kt) {
+        uint32_t mask;
+        if constexpr (KTAIL) mask = kt * BK + lchunk * 8 >= p.K ? kOutOfRange : 0u;
+        else mask = kt >= ke ? kOutOfRange : 0u;
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(base_a, 0, (!KTAIL && mask) ? 0 : bytes_a, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(base_b, 0, (!KTAIL && mask) ? 0 : bytes_b, kRsrcFlags);
+        const uint32_t lane_mask = KTAIL ? mask : 0u;
+#pragma unroll
+        for (int i = 0; i < PU; ++i) load_chunk(ra, lds + soff + i * 4096 + wave * 1024, voff_a[i] | lane_mask, kt * ROWB);
+#pragma unroll
+        for (int i = 0; i < PU; ++i) load_chunk(rb, lds + soff + UNIT + i * 4096 + wave * 1024, voff_b[i] | lane_mask, kt * ROWB);
+    };
+
+    const int frow = lane & 15, fq = lane >> 4;
+    int koff_a[KSUB], koff_w[KSUB];
+#pragma unroll
+    for (int kk = 0; kk < KSUB; ++kk) {
+        const int ko = ((kk * 4 + fq) ^ ((frow >> 1) & 7)) * 16;
+        koff_a[kk] = (wm * WROWS + frow) * ROWB + ko;
+        koff_w[kk] = UNIT + (wn * WROWS + frow) * ROWB + ko;
+    }
+    f32x4 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+    for (int s = 0; s < ST - 1; ++s) load_slab(s * SLAB, s);
+    int cur = 0, nxt = (ST - 1) * SLAB;
+    for (int kt = 0; kt < ke; ++kt) {
+        // slab kt has landed (this wave's part: all but the loads of the ST - 2 slabs behind it; the
+        // others' by the barrier), and every wave has the fragments of slab kt - 1 in registers
+        wait_loads_and_barrier<(ST - 2) * NL>();
+        load_slab(nxt, kt + ST - 1);
+#pragma unroll
+        for (int kk = 0; kk < KSUB; ++kk) {
+            bf16x8 xa[FM], wb[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) xa[i] = *reinterpret_cast<const bf16x8*>(lds + cur + koff_a[kk] + i * 16 * ROWB);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) wb[j] = *reinterpret_cast<const bf16x8*>(lds + cur + koff_w[kk] + j * 16 * ROWB);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[j], xa[i], acc[i][j], 0, 0, 0);
+        }
+        nxt = cur;
+        cur = cur + SLAB == ST * SLAB ? 0 : cur + SLAB;
+    }
+    wait_vmem_all();
+    __syncthreads();
+    gemm_epilogue<MI, MI>(p, acc, lds, m0, n0, wave, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Rectangular tiles: (32*FM) x (32*FN) per workgroup, a wave owns (16*FM) x (16*FN) as FM x FN
 // accumulators. One workgroup per CU means a launch costs whole rounds of 256 tiles; 4608 x 3072
 // (linear2 of the Flux block) is 216 tiles of 256 x 256, 0.84 of a round with 40 CUs idle, but
@@ -1246,6 +1345,17 @@ static void launch_tiled(GemmParams& p, hipStream_t st) {
     else hipLaunchKernelGGL((gemm_nt_ring_kernel<MI, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
 }
 
+template <int MI, int ST>
+static void launch_deep(GemmParams& p, hipStream_t st) {
+    constexpr int BM = 64 * MI;
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BM - 1) / BM;
+    p.group_m = 4;
+    const int grid = ((p.tiles_m * p.tiles_n + 7) / 8) * 8;
+    if (p.K % 64 == 0) hipLaunchKernelGGL((gemm_nt_deep_kernel<MI, ST, false>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+    else hipLaunchKernelGGL((gemm_nt_deep_kernel<MI, ST, true>), dim3(grid), dim3(kGemmThreads), 0, st, p);
+}
+
 // Rectangular tile shapes the host may pick: 288 x 192 and 256 x 192.
 template <int FM, int FN>
 static void launch_rect(GemmParams& p, hipStream_t st) {
@@ -1355,7 +1465,7 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
     const int64_t mid_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
     // 256-wide tiles once they fill most of the chip; below that 128-wide ones (two workgroups per
     // CU); problems with too few of those to give every second CU one are bound by the latency of
-    // the K loop and run on 64-wide tiles, four times as many workgroups.
+    // the K loop and run on 64-wide tiles with a deeper ring, four times as many workgroups.
     // Rectangular tiles (288 x 192 or 256 x 192) when both extents divide and their rounds come out
     // shorter than those of the other tiles. Measured at K = 3072: a round of square tiles 69 us, a
     // round of 288 x 192 tiles 62 us (0.84 of the work at 1.06 times the cost per flop), a launch on
@@ -1422,7 +1532,10 @@ extern "C" int flux_linear_bf16(const flux_linear_args* a, void* stream) {
             launch_tiled<2>(tail, st);
         }
     }
-    else if (mid_tiles <= 64) launch_tiled<1>(p, st);
+    // up to one round of 64-wide tiles at two workgroups per CU: the K loop's latency is the whole cost,
+    // and the kernel that keeps three slabs in flight wins (3072 x 3072 weights from HBM: 256 rows
+    // 39 -> 24 us, 512 rows 44 -> 35 us; from 768 rows on the 128-wide tiles are faster again)
+    else if (mid_tiles <= kGemmCUs / 2 && !(a->flags & FLUX_LINEAR_SHARED_GPU)) launch_deep<1, 4>(p, st);   // beside another stream: few, larger workgroups
     else if (!rect_if_cheaper(0.57 * static_cast<double>((mid_tiles + 2 * kGemmCUs - 1) / (2 * kGemmCUs)))) launch_tiled<2>(p, st);
     return check_launch("flux_linear_bf16");
 }
