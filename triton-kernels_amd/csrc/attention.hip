@@ -101,6 +101,7 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+#ifndef FLUX_ATTN_W64_D64_UNIT   // the 32-row kernel belongs to the main unit only
 // Slot of softmax unit g of a tile (see the kernel): units are spread evenly behind the max phase.
 constexpr int attn_unit_slot(int g, int qb_count, int nslot, int nunits) {
     return 5 * qb_count + g * (nslot - 9 * qb_count) / nunits;
@@ -446,6 +447,8 @@ __global__ __launch_bounds__(256, (QB == 1 ? 2 : 1)) void attn_fwd_pipe_kernel(A
     }
 }
 
+
+#endif  // FLUX_ATTN_W64_D64_UNIT
 
 // ------------------------------------------------------------------------------------------------
 // Head dim 128, 64 query rows per wave, one wave per SIMD, v_mfma_f32_16x16x32_bf16.
@@ -1130,16 +1133,10 @@ __device__ __forceinline__ void attn_w64_tile(const AttnParams& p, char* lds, co
 
 constexpr int w64_lds_bytes(int d) { return 8 * 64 * 2 * d; }  // K ring and V ring of four 64-key tiles
 
-template <int D, int QB, int NW>
-__global__ __launch_bounds__(64 * NW, 1) void attn_fwd_w64_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(1024))) char lds[w64_lds_bytes(D)];
-    attn_w64_tile<D, QB, NW>(p, lds, blockIdx.x, gridDim.x);
-}
-
 // Both tile sizes in one launch: blocks [0, n4) take 256-row tiles of p4, the rest 192-row tiles of
 // p3. Workgroups are handed out in order, so the 192-row tiles start on each CU as it finishes its
 // 256-row tile, with no launch boundary in between. n4 and the remainder are multiples of eight, so
-// a block's XCD is the same counted from either start.
+// a block's XCD is the same counted from either start. A launch of 256-row tiles only has n4 = grid.
 template <int D>
 __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel_pair(AttnParams p4, AttnParams p3, int n4) {
     __shared__ __attribute__((aligned(1024))) char lds[w64_lds_bytes(D)];
@@ -1147,6 +1144,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_w64_kernel_pair(AttnParams p4
     else attn_w64_tile<D, 3, 4>(p3, lds, static_cast<int>(blockIdx.x) - n4, static_cast<int>(gridDim.x) - n4);
 }
 
+#ifndef FLUX_ATTN_W64_D64_UNIT
 template <int D, int QB, int BN>
 static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
     p.n_qtiles = (p.L + 128 * QB - 1) / (128 * QB);
@@ -1154,6 +1152,8 @@ static void attn_launch_pipe(AttnParams& p, int64_t BH, hipStream_t st) {
     const int grid = ((p.total_tiles + 7) / 8) * 8;
     hipLaunchKernelGGL((attn_fwd_pipe_kernel<D, QB, BN>), dim3(grid), dim3(256), 0, st, p);
 }
+
+#endif
 
 constexpr int64_t kW64MinTiles = 128;
 
@@ -1249,11 +1249,20 @@ static void attn_launch_w64(AttnParams& p, int64_t BH, hipStream_t st) {
         }
     }
     const int g = attn_w64_part(p, BH, n256, n256, 0, 0);
-    if (g > 0) hipLaunchKernelGGL((attn_fwd_w64_kernel<D, 4, 4>), dim3(g), dim3(256), 0, st, p);
+    if (g > 0) hipLaunchKernelGGL(attn_fwd_w64_kernel_pair<D>, dim3(g), dim3(256), 0, st, p, p, g);
 }
+
+// The head-dim-64 instantiation of the 64-row kernels is compiled as a unit of its own
+// (attention_d64.hip includes this file with FLUX_ATTN_W64_D64_UNIT defined): the unrolled loop
+// bodies take minutes to compile, and the two head dims compile side by side.
+void attn_launch_w64_d64(AttnParams& p, int64_t BH, hipStream_t st);
+#ifdef FLUX_ATTN_W64_D64_UNIT
+void attn_launch_w64_d64(AttnParams& p, int64_t BH, hipStream_t st) { attn_launch_w64<64>(p, BH, st); }
+#endif
 
 }  // namespace flux
 
+#ifndef FLUX_ATTN_W64_D64_UNIT
 using namespace flux;
 
 static bool view_ok(const void* ptr, int64_t sb, int64_t sh, int64_t sl) {
@@ -1292,7 +1301,8 @@ extern "C" int flux_attention_fwd_bf16(const flux_attn_args* a, void* stream) {
         attn_launch_plain(p, BH, a->D, st);
     } else if (a->D == 128 && tiles256 >= kW64MinTiles) attn_launch_w64<128>(p, BH, st);
     else if (a->D == 128) attn_launch_pipe<128, 1, 64>(p, BH, st);
-    else if (tiles256 >= kW64MinTiles) attn_launch_w64<64>(p, BH, st);
+    else if (tiles256 >= kW64MinTiles) attn_launch_w64_d64(p, BH, st);
     else attn_launch_pipe<64, 1, 64>(p, BH, st);
     return check_launch("flux_attention_fwd_bf16");
 }
+#endif  // FLUX_ATTN_W64_D64_UNIT
