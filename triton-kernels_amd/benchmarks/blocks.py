@@ -82,6 +82,7 @@ def main(argv=None):
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--runs", type=int, default=100)
     ap.add_argument("--atol", type=float, default=0.1)
+    ap.add_argument("--no-baseline", action="store_true", help="skip timing the plain PyTorch block (for kernel traces of the HIP one)")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("blocks.py needs a GPU: the HIP kernels have no CPU path")
@@ -91,7 +92,8 @@ def main(argv=None):
                          args.hidden, args.heads, dev)
     worst = compare(plain, hip, inputs, args.atol)
     print(f"max |hip - baseline| = {worst:.4f} (atol {args.atol})")
-    print(f"baseline block time: {time_block(plain, inputs, args.warmup, args.runs):.3f} ms per pass")
+    if not args.no_baseline:
+        print(f"baseline block time: {time_block(plain, inputs, args.warmup, args.runs):.3f} ms per pass")
     print(f"     hip block time: {time_block(hip, inputs, args.warmup, args.runs):.3f} ms per pass")
 
 
